@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-token forward path: LLaMA-7B-shape f16 batch-1 greedy decode on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline]
+
+A "step" is one decoded token: the full token step (5 kernels per layer + output head) plus the greedy
+pick, fed on the device with the previous step's token.  The workload is config 1 of the benchmark
+definition: 128 synthetic prompt ids, then K (default 256) greedy tokens; random-init weights N(0, 0.02)
+from the repo's counter-based generator, seed 0.  Prints ONE JSON line.
+
+Nothing here reads the reference checkout; the CPU oracle is used only for the `cpu_baseline` leg.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+CONFIGS = {
+    # name: (dim, n_layers, n_heads, ffn_hidden, vocab, n_prompt, default decode steps)
+    "c0": (1024, 8, 16, 2816, 32000, 16, 64),
+    "c1": (4096, 32, 32, 11008, 32000, 128, 256),
+    "c2": (5120, 40, 40, 13824, 32000, 2048, 128),
+    "c4": (8192, 80, 64, 22016, 32000, 256, 128),
+}
+
+
+def cpu_baseline(model, dim, n_layers, n_heads, ffn, vocab, n_prompt=8, n_decode=16):
+    """The CPU oracle (restatement of rllama's AVX2 path) on this host's cores, on the same weights.
+
+    Times `n_decode` single-token forwards after an `n_prompt`-token prompt, ms/token defined like
+    rllama_main.rs:890-894 (prefill call excluded), threads = the cores this process may use.
+    """
+    import oracle
+    import rllama_amd as ra
+
+    cores = len(os.sched_getaffinity(0))
+    try:
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    except ValueError:
+        pass
+    oracle.set_threads(cores)
+    oracle.set_reference_threading(True)
+    om = oracle.Model(dim, n_layers, n_heads, ffn, vocab, n_prompt + n_decode + 1, 1e-6, True)
+    shapes = {ra.WQ: (dim, dim), ra.WK: (dim, dim), ra.WV: (dim, dim), ra.WO: (dim, dim), ra.W1: (ffn, dim), ra.W3: (ffn, dim), ra.W2: (dim, ffn)}
+    for kind in (ra.TOK_EMB, ra.OUTPUT):
+        om.set_tensor(kind, 0, model.get_tensor(kind, 0, vocab, dim, as_f16_bits=True))
+    om.set_tensor(ra.NORM, 0, model.get_tensor(ra.NORM, 0, 1, dim))
+    for l in range(n_layers):
+        for kind, (r, c) in shapes.items():
+            om.set_tensor(kind, l, model.get_tensor(kind, l, r, c, as_f16_bits=True))
+        for kind in (ra.ATTN_NORM, ra.FFN_NORM):
+            om.set_tensor(kind, l, model.get_tensor(kind, l, 1, dim))
+    prompt = ra.synth_tokens(0, n_prompt, 3, vocab)
+    oc = om.make_caches()
+    toks = list(prompt)
+    t0 = time.perf_counter()
+    logits = om.forward(toks, 0, oc)
+    t_first = time.perf_counter() - t0
+    per = []
+    for _ in range(n_decode):
+        tok, _, _ = oracle.sample_greedy(logits)
+        toks.append(tok)
+        t0 = time.perf_counter()
+        logits = om.forward(toks[-1:], len(toks) - 1, oc)
+        per.append(time.perf_counter() - t0)
+    ms = 1e3 * float(np.mean(per))
+    return {
+        "value": round(ms, 2), "unit": "ms/token", "cores": cores, "kind": "port",
+        "sample": f"same shape and weights, f16 mode, {n_prompt} prompt + {n_decode} greedy decode tokens "
+                  f"(first call {1e3 * t_first:.0f} ms excluded)",
+        "tokens_per_s": round(1e3 / ms, 3),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel-iters", type=int, default=320)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (batch-1 decode of one model resident in one device's HBM); "
+              f"--gpus {args.gpus} is not supported.", file=sys.stderr)
+        return 2
+
+    import rllama_amd as ra
+
+    dim, n_layers, n_heads, ffn, vocab, n_prompt, dflt_steps = CONFIGS[args.config]
+    K = args.steps if args.steps is not None else dflt_steps
+    W = max(0, args.warmup)
+    max_seq = n_prompt + max(K, W) + 1
+
+    ctx = ra.Context(0, verbose=False)
+    info = ctx.device_info()
+    ds = ra.DataSettings(ctx).force_f16()
+    model = ra.Transformer(ctx, dim, n_layers, n_heads, ffn, vocab, max_seq, 1e-6, ds)
+    model.fill_synthetic(seed=0, std=0.02)
+    prompt = ra.synth_tokens(0, n_prompt, 3, vocab)
+
+    # ---- warmup: W untimed decode steps (own caches, same prompt) ----
+    cw = model.make_caches()
+    model.generate_greedy(prompt, 1, cw)
+    if W > 0:
+        model.decode_greedy(W, cw)
+    cw.free()
+
+    # ---- timed region: exactly K decode steps after the prompt ----
+    caches = model.make_caches()
+    first_ids, ms_prompt, _ = model.generate_greedy(prompt, 1, caches)   # prompt pass + first token (untimed)
+    ctx.sync()
+    t0 = time.perf_counter()
+    ids, ms_events = model.decode_greedy(K, caches)                      # K token steps, no host round trip
+    ctx.sync()
+    wall_ms = 1e3 * (time.perf_counter() - t0)
+    ms_per_step = wall_ms / K
+
+    # algorithmic HBM bytes of the K steps: weights once per token + KV rows read + written
+    T_values = [n_prompt + i + 1 for i in range(K)]                      # sequence length seen by step i
+    step_bytes = [model.decode_bytes(T) for T in T_values]
+    mean_bytes = float(np.mean(step_bytes))
+    e2e_gbps = mean_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-kernel timing (HIP events on the launch stream, weights cycled over all layers) ----
+    T_mid = n_prompt + K // 2
+    kernels = {}
+    for which, name in enumerate(ra.Transformer.STEP_KERNELS):
+        us, nbytes = model.time_kernel(which, T_mid, args.kernel_iters if which != 5 else max(20, args.kernel_iters // 8), caches)
+        kernels[name] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3)}
+    dom = "w13_silu"  # ffn_norm + w1|w3 + SiLU*gate: the largest share of the bytes of a token step
+    roofline = {
+        "bound": "hbm", "kernel": "gemv_kernel<f16 weights, f16 x, SiLU epilogue> (" + dom + ")",
+        "achieved": kernels[dom]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": round(kernels[dom]["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+        "algorithmic_bytes_per_launch": kernels[dom]["bytes"], "us_per_launch": kernels[dom]["us"],
+    }
+
+    # ---- isolated GEMV microbench: [11008 x 4096] and [4096 x 11008] f16 against fp32 x, >1 GB of weights cycled ----
+    micro = {}
+    if args.config == "c1":
+        for rows, k in ((11008, 4096), (4096, 11008)):
+            us = ctx.time_gemv(rows, k, ra.TensorDType.Float16, False, False, n_buffers=12, iters=240)
+            nb = rows * k * 2 + k * 4 + rows * 4
+            micro[f"{rows}x{k}"] = {"us": round(us, 2), "bytes": nb, "GBps": round(nb / us / 1e3, 1), "frac": round(nb / us / 1e3 / HBM_PEAK_GBPS, 3)}
+
+    out = {
+        "metric": f"ms/token, LLaMA-{ {'c0': 'tiny', 'c1': '7B', 'c2': '13B', 'c4': '65B'}[args.config] }-shape f16 batch-1 greedy decode, 1 MI355X",
+        "value": round(ms_per_step, 4), "unit": "ms/token", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 weights/KV, fp32 accumulate", "data": "synthetic (random-init N(0,0.02) weights seed 0, synthetic token ids)",
+        "config": {"workload": f"{args.config}: dim {dim}, {n_layers} layers, {n_heads} heads, ffn {ffn}, vocab {vocab}; "
+                               f"{n_prompt} prompt ids then {K} greedy decode tokens, batch 1", "max_seq_len": max_seq},
+        "tokens_per_s": round(1e3 / ms_per_step, 2),
+        "ms_per_token_hip_events": round(ms_events / K, 4),
+        "ms_prompt_pass": round(ms_prompt, 2),
+        "hbm_GBps_end_to_end": round(e2e_gbps, 1),
+        "hbm_frac_end_to_end": round(e2e_gbps / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes_per_token": int(mean_bytes),
+        "roofline": roofline,
+        "kernels": kernels,
+        "gemv_microbench": micro,
+        "device": info["name"],
+        "first_tokens": [int(first_ids[0])] + [int(t) for t in ids[:7]],
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(model, dim, n_layers, n_heads, ffn, vocab)
+    else:
+        out["cpu_baseline"] = None
+    caches.free()
+    model.free()
+    ctx.close()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

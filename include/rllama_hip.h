@@ -1,0 +1,217 @@
+/*
+ * rllama_hip.h -- C ABI of librllama_hip.so: rllama's per-token transformer forward path on one
+ * MI355X (gfx950), weights and KV cache resident in HBM.
+ *
+ * This is the seam rllama's `opencl` Cargo feature occupies (Cargo.toml:42-44; Tensor.opencl_data,
+ * src/tensor.rs:99-102; DataSettings, src/transformer.rs:38-109).  A Rust host binds these symbols
+ * from an `extern "C"` block; nothing here needs a C++ or torch type.
+ *
+ * Conventions
+ *   - every function returns 0 on success or a nonzero rlh_status; rlh_last_error() gives the text of
+ *     the calling thread's most recent failure (the reference's OpenCLError strings,
+ *     src/tensor_opencl_support.rs:77-83, play this role);
+ *   - handles are opaque; a handle belongs to the context that made it;
+ *   - all calls on one context are serialised by the library (the reference serialises on a
+ *     `programs.write()` lock and one in-order queue, src/tensor_opencl_support.rs:120, :322);
+ *   - host pointers are only read/written during the call unless stated otherwise;
+ *   - there is no CPU fallback: without a usable HIP device rlh_init fails and nothing else works.
+ *
+ * Citations `file:line` are into the reference checkout (Noeda/rllama).
+ */
+#ifndef RLLAMA_HIP_H
+#define RLLAMA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    RLH_OK = 0,
+    RLH_ERR_INVALID = 1,      /* bad argument / shape; where the reference panics on a shape assert */
+    RLH_ERR_NO_DEVICE = 2,    /* no HIP device / ordinal out of range (OpenCLError::OpenCLDeviceListError) */
+    RLH_ERR_HIP = 3,          /* a HIP runtime call failed (OpenCLError::OpenCL) */
+    RLH_ERR_OOM = 4,          /* device allocation failed */
+    RLH_ERR_STATE = 5,        /* model not fully loaded, caches of another model, sequence too long ... */
+    RLH_ERR_UNSUPPORTED = 6   /* arch is not gfx950, or a dtype the reference does not offload either */
+} rlh_status;
+
+typedef enum { RLH_F16 = 0, RLH_F32 = 1 } rlh_dtype;   /* TensorDType (src/tensor.rs:50-54) */
+
+/* Weight names: src/transformer.rs:297-304, 405-412, 490-503, 595-614; src/embedding.rs:18 */
+typedef enum {
+    RLH_TOK_EMB = 0,     /* tok_embeddings.weight            [vocab x dim]  */
+    RLH_WQ = 1,          /* layers.i.attention.wq.weight     [dim x dim]    */
+    RLH_WK = 2,
+    RLH_WV = 3,
+    RLH_WO = 4,
+    RLH_W1 = 5,          /* layers.i.feed_forward.w1.weight  [ffn x dim]    */
+    RLH_W2 = 6,          /* layers.i.feed_forward.w2.weight  [dim x ffn]    */
+    RLH_W3 = 7,          /* layers.i.feed_forward.w3.weight  [ffn x dim]    */
+    RLH_ATTN_NORM = 8,   /* layers.i.attention_norm.weight   [dim]          */
+    RLH_FFN_NORM = 9,    /* layers.i.ffn_norm.weight         [dim]          */
+    RLH_NORM = 10,       /* norm.weight                      [dim]          */
+    RLH_OUTPUT = 11      /* output.weight                    [vocab x dim]  */
+} rlh_tensor_kind;
+
+typedef struct rlh_ctx rlh_ctx;
+typedef struct rlh_model rlh_model;
+typedef struct rlh_caches rlh_caches;
+typedef struct rlh_tensor rlh_tensor;
+typedef struct rlh_event rlh_event;
+
+/* ------------------------------------------------------------------------------------------------
+ * Context.  Replaces OpenCL::new(verbose, nth_device) (src/tensor_opencl_support.rs:86-128), called
+ * from src/rllama_main.rs:182-199.  Fails (no fallback) if the ordinal does not name a gfx950 device.
+ * ---------------------------------------------------------------------------------------------- */
+int  rlh_init(int device_ordinal, int verbose, rlh_ctx **out);
+void rlh_shutdown(rlh_ctx *ctx);
+/* OpenCL::flush (src/tensor_opencl_support.rs:130) / Tensor::finish (src/tensor.rs:2198-2206): returns
+ * when all work queued on the context has completed. */
+int  rlh_sync(rlh_ctx *ctx);
+const char *rlh_last_error(void);
+/* Device facts for reports: name (<= cap bytes incl. NUL), compute units, total HBM bytes. */
+int  rlh_device_info(rlh_ctx *ctx, char *name, int cap, int *compute_units, uint64_t *hbm_bytes);
+
+/* ------------------------------------------------------------------------------------------------
+ * Model.  Replaces Transformer::from_unpickled (src/transformer.rs:242-326) + the per-tensor
+ * to_f16()/to_gpu_inplace() calls (src/transformer.rs:508-525, 624-644).
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct {
+    int32_t dim;                /* params.json "dim"        (src/model_params.rs:3-14) */
+    int32_t n_layers;           /* "n_layers" */
+    int32_t n_heads;            /* "n_heads"; dim % n_heads == 0 (src/transformer.rs:252) */
+    int32_t ffn_hidden;         /* rows of w1 as stored; not a params.json field */
+    int32_t vocab_size;         /* "vocab_size" */
+    int32_t max_seq_len;        /* --max-seq-len (src/rllama_main.rs:247): RoPE table and cache length */
+    double  norm_eps;           /* "norm_eps" */
+    int32_t force_f16;          /* --f16, DataSettings::force_f16 (src/transformer.rs:105-108): 1 = f16
+                                   projection weights, f16 KV cache and the f16 rounding points of
+                                   src/transformer.rs:665-668, 537-540, 563-565, 795;
+                                   0 = f32 weights, f32 KV cache, no rounding anywhere */
+    float   percentage_to_gpu;  /* --percentage-to-gpu; clamped like src/transformer.rs:91-103.  On one
+                                   288 GB device every layer is resident: see rlh_model_layers_on_gpu */
+} rlh_model_params;
+
+int  rlh_model_create(rlh_ctx *ctx, const rlh_model_params *params, rlh_model **out);
+void rlh_model_free(rlh_model *model);
+/* Copies one weight from host memory into HBM.  `host` is dense row-major [rows x cols] of src_dtype
+ * (f16 = IEEE binary16 bits, as in consolidated.NN/data/<k>; src/tensor.rs:2498-2538).  Norm vectors
+ * are [1 x dim].  layer is ignored for TOK_EMB / NORM / OUTPUT.  Under force_f16 an f32 source is
+ * rounded to f16 like Tensor::to_f16 (src/tensor.rs:2281-2314).  The host buffer is free on return. */
+int  rlh_model_set_tensor(rlh_model *model, int kind, int layer, const void *host, int rows, int cols, int src_dtype);
+/* Reads a stored weight back as dst_dtype [rows x cols]: RLH_F32 gives what Tensor::to_f32 of it would hold,
+ * RLH_F16 the IEEE binary16 bits (exact for f16 storage, Tensor::to_f16 rounding for f32 storage). */
+int  rlh_model_get_tensor(rlh_model *model, int kind, int layer, void *host_out, int rows, int cols, int dst_dtype);
+/* Fills every weight on the device from the counter-based generator in synth.h: projection matrices,
+ * embedding and head i.i.d. N(0, std^2) rounded to f16, norm weights 1.0.  Bit-identical to
+ * rlh_synth_normal_f16 on the host.  (No reference counterpart: the reference only loads files.) */
+int  rlh_model_fill_synthetic(rlh_model *model, uint64_t seed, double std);
+/* The layer split rule of src/transformer.rs:262-279: last_layer_on_gpu = round(p * (n_layers - 1)).
+ * Reports it; all layers run on the device regardless (nothing is left on the host). */
+int  rlh_model_layers_on_gpu(const rlh_model *model, int *last_layer_on_gpu);
+/* Bytes of HBM one decode step must read at sequence length T: weights + KV (the roofline's numerator). */
+int  rlh_model_decode_bytes(const rlh_model *model, int T, uint64_t *bytes);
+
+/* ------------------------------------------------------------------------------------------------
+ * KV caches.  TransformerCaches / AttentionCache (src/transformer.rs:111-214).
+ * ---------------------------------------------------------------------------------------------- */
+int  rlh_caches_create(rlh_model *model, rlh_caches **out);                 /* make_caches :328-341 (zero filled) */
+int  rlh_caches_true_clone(const rlh_caches *src, rlh_caches **out);        /* true_clone  :207-213 */
+int  rlh_caches_shift_left(rlh_caches *caches, int shifts);                 /* shift_left  :201-205 */
+void rlh_caches_free(rlh_caches *caches);
+/* Test hook: (layer, head) cache contents as f32 [head_dim x max_seq_len], position along columns, the
+ * reference's own orientation (src/transformer.rs:143-154).  which: 0 = K, 1 = V. */
+int  rlh_caches_read(const rlh_caches *caches, int layer, int head, int which, float *host_out);
+
+/* ------------------------------------------------------------------------------------------------
+ * Forward.  Transformer::forward(tokens, start_pos, caches) -> logits[vocab] (src/transformer.rs:343-383).
+ * Valid calls are the reference's: any n >= 1 at start_pos == 0, n == 1 at start_pos > 0 (the mask of
+ * :350-357 only fits start_pos == 0), start_pos + n <= max_seq_len.  logits_out: vocab floats on the host.
+ * ---------------------------------------------------------------------------------------------- */
+int  rlh_forward(rlh_model *model, rlh_caches *caches, const int32_t *tokens, int n, int start_pos, float *logits_out);
+/* forward + TokenSampler::sample with top_k = 1, temperature = 1, repetition_penalty = 1
+ * (src/token_sampler.rs:83-174; its loops over 0..logits.rows() only ever touch token 0, whose logit
+ * becomes 0.0): the argmax runs on the device, only the id crosses PCIe. */
+int  rlh_forward_greedy(rlh_model *model, rlh_caches *caches, const int32_t *tokens, int n, int start_pos, int32_t *next_token);
+/* The token loop of command_line_inference (src/rllama_main.rs:821-897) at top_k = 1: one forward over
+ * the prompt, then one single-token forward per new token, each fed the previous argmax on the device.
+ * out_tokens receives n_new ids.  ms_first / ms_per_token (may be NULL) are measured with HIP events
+ * on the launch stream and follow src/rllama_main.rs:890-894, 908-917 (first call apart, then the mean
+ * over the remaining steps). */
+int  rlh_generate_greedy(rlh_model *model, rlh_caches *caches, const int32_t *prompt, int n_prompt, int n_new,
+                         int32_t *out_tokens, float *ms_first, float *ms_per_token);
+
+/* Continues the greedy token loop from where rlh_forward_greedy / rlh_generate_greedy / rlh_decode_greedy left
+ * it (the last sampled id and its position are still on the device): n_steps further single-token forwards,
+ * no host round trip in between.  out_tokens receives n_steps ids; ms_total (may be NULL) is the HIP-event
+ * time of the n_steps steps on the launch stream. */
+int  rlh_decode_greedy(rlh_model *model, rlh_caches *caches, int n_steps, int32_t *out_tokens, float *ms_total);
+
+/* ------------------------------------------------------------------------------------------------
+ * Op level.  Mirrors OpenCLTensor (src/tensor_opencl_support.rs:134-405) so that a host Tensor can
+ * offload single ops, and so that each kernel can be checked alone.  Tensors are dense row-major.
+ * ---------------------------------------------------------------------------------------------- */
+/* OpenCL::data_u16_to_gpu (:134-169), generalised to f32.  cols_capacity = row stride of the HOST buffer in
+ * elements (src/tensor.rs:192-222); the device copy is dense. */
+int  rlh_tensor_upload(rlh_ctx *ctx, const void *host, int rows, int cols, int cols_capacity, int dtype, rlh_tensor **out);
+int  rlh_tensor_alloc(rlh_ctx *ctx, int rows, int cols, int dtype, rlh_tensor **out);   /* zero filled */
+/* OpenCLTensor::data_u16_from_gpu (:198-212): asynchronous read; *ev (may be NULL = wait inside) must be
+ * waited on before `host` is read.  Host row stride = cols_capacity. */
+int  rlh_tensor_download(rlh_tensor *t, void *host, int cols_capacity, rlh_event **ev);
+void rlh_tensor_free(rlh_tensor *t);
+int  rlh_tensor_shape(const rlh_tensor *t, int *rows, int *cols, int *dtype);
+int  rlh_event_wait(rlh_event *ev);                               /* OpenCLEvent::wait (:409-411); frees the event */
+/* HIP-event timing on the launch stream (for measurements). */
+int  rlh_event_record(rlh_ctx *ctx, rlh_event **out);
+int  rlh_event_elapsed_ms(rlh_event *start, rlh_event *stop, float *ms);   /* waits for stop */
+void rlh_event_free(rlh_event *ev);
+
+int  rlh_copy_inplace(rlh_tensor *dst, const rlh_tensor *src);                       /* :215-232 */
+int  rlh_transpose_from(rlh_tensor *dst, const rlh_tensor *src);                     /* :234-256 */
+int  rlh_hadamard_product_inplace(rlh_tensor *dst, const rlh_tensor *src);           /* :258-281; f16: result rounded to f16 */
+int  rlh_silu_inplace(rlh_tensor *t);                                                /* :283-299 */
+/* OpenCLTensor::matrix_mul_inplace_transposed(self, src, other) (:301-405): dst[r, c] = sum_k src[r, k] * other[c, k].
+ * src [n x k], other [m x k], dst [n x m].  f16 operands give an f16-rounded dst (as src/tensor.rs:1623-1643);
+ * f32 operands give f32.  src and other must share a dtype; dst has it too.  n == 1 takes the GEMV kernel,
+ * n > 1 the MFMA GEMM (f16) or the tiled fp32 kernel. */
+int  rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tensor *src, const rlh_tensor *other);
+/* Decode GEMV with the rounding switches of the fused path: y[c] = sum_k x[k] * W[c, k]; x f32 [1 x k]
+ * (rounded to f16 first if round_x), W f16 or f32 [m x k], y f32 [1 x m] (rounded to f16 precision if round_y). */
+int  rlh_gemv(rlh_tensor *y, const rlh_tensor *w, const rlh_tensor *x, int round_x, int round_y);
+/* RMSNorm::forward (src/transformer.rs:476-480) per row; x, y f32 [n x d], w f32 [1 x d]; round_y = f16 rounding point. */
+int  rlh_rmsnorm(rlh_tensor *y, const rlh_tensor *x, const rlh_tensor *w, double eps, int round_y);
+/* apply_rotary_emb (src/transformer.rs:823-856) on one [n_heads x head_dim] f32 row at position pos, in place. */
+int  rlh_rope_inplace(rlh_tensor *x, int n_heads, int head_dim, int pos);
+
+/* ------------------------------------------------------------------------------------------------
+ * Measurement aids (no reference counterpart; src/benches/benchmark.rs times the CPU/OpenCL ops with criterion).
+ * Both time `iters` back-to-back launches with HIP events on the launch stream.
+ * ---------------------------------------------------------------------------------------------- */
+/* One kernel of the token step, cycling through the layers so that every launch streams different weights.
+ * which: 0 = attention_norm + wq|wk|wv + RoPE + cache write, 1 = single-query attention at sequence length T,
+ * 2 = wo + residual, 3 = ffn_norm + w1|w3 + SiLU*gate, 4 = w2 + residual, 5 = final norm + output head.
+ * bytes_per_launch (may be NULL): the algorithmic bytes of one launch (weights once + vectors). */
+int  rlh_model_time_kernel(rlh_model *model, rlh_caches *caches, int which, int T, int iters, float *us_per_launch,
+                           uint64_t *bytes_per_launch);
+/* Isolated GEMV y = W x, W [rows x k] of w_dtype, x f32, cycling through n_buffers distinct weight buffers
+ * (choose n_buffers * rows * k * elem size well above the 256 MB last-level cache). */
+int  rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int round_x, int round_y, int n_buffers, int iters,
+                   float *us_per_launch);
+
+/* ------------------------------------------------------------------------------------------------
+ * Synthetic inputs (host side; usable without a device).  See synth.h.
+ * ---------------------------------------------------------------------------------------------- */
+void rlh_synth_normal_f16(uint64_t seed, int kind, int layer, uint64_t first_index, uint64_t count, double std, uint16_t *out);
+void rlh_synth_tokens(uint64_t seed, uint64_t first_index, uint64_t count, int32_t lo, int32_t hi, int32_t *out);
+
+/* ABI version of this header. */
+int  rlh_abi_version(void);
+#define RLH_ABI_VERSION 1
+
+#ifdef __cplusplus
+}
+#endif
+#endif

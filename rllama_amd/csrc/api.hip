@@ -1,0 +1,1242 @@
+// api.hip -- the C ABI of librllama_hip.so (include/rllama_hip.h): context, HBM-resident model and KV
+// caches, the token-step launch sequence, and the op-level entry points.
+//
+// Structure mirrors what it replaces in the reference (Noeda/rllama): OpenCL (tensor_opencl_support.rs:40-58)
+// -> rlh_ctx; Transformer (transformer.rs:17-34) -> rlh_model; TransformerCaches (transformer.rs:111-113)
+// -> rlh_caches; OpenCLTensor (tensor_opencl_support.rs:23-38) -> rlh_tensor.
+#include "../../include/rllama_hip.h"
+#include "kernels.h"
+#include "synth.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+using namespace rlh;
+
+// ------------------------------------------------------------------------------------------------
+// errors
+// ------------------------------------------------------------------------------------------------
+static thread_local std::string g_last_error;
+
+static int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                                     \
+    do {                                                                                                  \
+        hipError_t _e = (expr);                                                                           \
+        if (_e != hipSuccess) {                                                                           \
+            return fail(_e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "%s failed: %s (%s:%d)",   \
+                        #expr, hipGetErrorString(_e), __FILE__, __LINE__);                                \
+        }                                                                                                 \
+    } while (0)
+
+extern "C" const char *rlh_last_error(void) { return g_last_error.c_str(); }
+extern "C" int rlh_abi_version(void) { return RLH_ABI_VERSION; }
+
+// ------------------------------------------------------------------------------------------------
+// objects
+// ------------------------------------------------------------------------------------------------
+struct rlh_ctx {
+    int device = 0;
+    int verbose = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t prop;
+    std::recursive_mutex mu;
+};
+
+struct Weight {
+    void *p = nullptr;
+    int rows = 0, cols = 0;
+    int f16 = 0;
+    bool loaded = false;
+    size_t bytes() const { return (size_t)rows * cols * (f16 ? 2 : 4); }
+};
+
+struct Layer {
+    Weight wqkv; // rows [0,d) wq, [d,2d) wk, [2d,3d) wv: one fused GEMV streams all three
+    bool q_loaded = false, k_loaded = false, v_loaded = false;
+    Weight wo, w1, w2, w3, attn_norm, ffn_norm;
+};
+
+struct rlh_model {
+    rlh_ctx *ctx = nullptr;
+    rlh_model_params prm;
+    int head_dim = 0;
+    int last_layer_on_gpu = 0;
+    Weight tok_emb, norm, output;
+    std::vector<Layer> layers;
+    float2 *freqs = nullptr;
+    // activations of one token step
+    float *x = nullptr, *q = nullptr, *att = nullptr, *mh = nullptr, *logits = nullptr;
+    DecodeState *state = nullptr;
+    int32_t *out_tokens = nullptr;
+    int out_cap = 0;
+    int32_t *prompt_dev = nullptr;
+    int prompt_cap = 0;
+    float *attn_ws = nullptr;
+    unsigned int *attn_counters = nullptr;
+    int max_splits = 16;
+    int stream_weights = 1;
+    // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
+    int next_pos = -1;
+    rlh_caches *greedy_caches = nullptr;
+};
+
+struct rlh_caches {
+    rlh_model *model = nullptr;
+    void *k = nullptr, *v = nullptr;
+    size_t bytes_each = 0;
+    int f16 = 0;
+};
+
+struct rlh_tensor {
+    rlh_ctx *ctx = nullptr;
+    void *p = nullptr;
+    int rows = 0, cols = 0, dtype = RLH_F16;
+    size_t esize() const { return dtype == RLH_F16 ? 2 : 4; }
+    size_t count() const { return (size_t)rows * cols; }
+};
+
+struct rlh_event {
+    rlh_ctx *ctx = nullptr;
+    hipEvent_t ev = nullptr;
+};
+
+struct CtxLock {
+    std::lock_guard<std::recursive_mutex> g;
+    explicit CtxLock(rlh_ctx *c) : g(c->mu) { (void)hipSetDevice(c->device); }
+};
+
+// ------------------------------------------------------------------------------------------------
+// context
+// ------------------------------------------------------------------------------------------------
+extern "C" int rlh_init(int device_ordinal, int verbose, rlh_ctx **out) {
+    if (!out) return fail(RLH_ERR_INVALID, "rlh_init: out is NULL");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        return fail(RLH_ERR_NO_DEVICE, "rlh_init: no HIP device (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    }
+    if (device_ordinal < 0 || device_ordinal >= count) {
+        return fail(RLH_ERR_NO_DEVICE, "rlh_init: device ordinal %d out of range (%d devices)", device_ordinal, count);
+    }
+    rlh_ctx *c = new rlh_ctx();
+    c->device = device_ordinal;
+    c->verbose = verbose;
+    if ((e = hipSetDevice(device_ordinal)) != hipSuccess || (e = hipGetDeviceProperties(&c->prop, device_ordinal)) != hipSuccess) {
+        delete c;
+        return fail(RLH_ERR_HIP, "rlh_init: %s", hipGetErrorString(e));
+    }
+    if (strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
+        int rc = fail(RLH_ERR_UNSUPPORTED, "rlh_init: device %d is %s; this library holds gfx950 code only", device_ordinal,
+                      c->prop.gcnArchName);
+        delete c;
+        return rc;
+    }
+    if ((e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking)) != hipSuccess) {
+        delete c;
+        return fail(RLH_ERR_HIP, "rlh_init: hipStreamCreate: %s", hipGetErrorString(e));
+    }
+    if (verbose) {
+        fprintf(stderr, "rllama_hip: device %d %s (%s), %d CUs, %.1f GB HBM\n", device_ordinal, c->prop.name, c->prop.gcnArchName,
+                c->prop.multiProcessorCount, (double)c->prop.totalGlobalMem / 1e9);
+    }
+    *out = c;
+    return RLH_OK;
+}
+
+extern "C" void rlh_shutdown(rlh_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipStreamDestroy(ctx->stream);
+    }
+    delete ctx;
+}
+
+extern "C" int rlh_sync(rlh_ctx *ctx) {
+    if (!ctx) return fail(RLH_ERR_INVALID, "rlh_sync: ctx is NULL");
+    CtxLock lock(ctx);
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_device_info(rlh_ctx *ctx, char *name, int cap, int *compute_units, uint64_t *hbm_bytes) {
+    if (!ctx) return fail(RLH_ERR_INVALID, "rlh_device_info: ctx is NULL");
+    if (name && cap > 0) snprintf(name, (size_t)cap, "%s (%s)", ctx->prop.name, ctx->prop.gcnArchName);
+    if (compute_units) *compute_units = ctx->prop.multiProcessorCount;
+    if (hbm_bytes) *hbm_bytes = (uint64_t)ctx->prop.totalGlobalMem;
+    return RLH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// model
+// ------------------------------------------------------------------------------------------------
+static void free_weight(Weight &w) {
+    if (w.p) (void)hipFree(w.p);
+    w.p = nullptr;
+}
+
+static int alloc_weight(Weight &w, int rows, int cols, int f16) {
+    w.rows = rows;
+    w.cols = cols;
+    w.f16 = f16;
+    HIP_TRY(hipMalloc(&w.p, w.bytes()));
+    return RLH_OK;
+}
+
+static float clamp_percentage(float p) {
+    // DataSettings::percentage_to_gpu (transformer.rs:91-103)
+    if (p >= 1.0f) p = 1.0f;
+    if (p < 0.0f) p = 0.0f;
+    if (std::isnan(p)) p = 0.0f;
+    return p;
+}
+
+extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_model **out) {
+    if (!ctx || !prm || !out) return fail(RLH_ERR_INVALID, "rlh_model_create: NULL argument");
+    *out = nullptr;
+    if (prm->dim <= 0 || prm->n_layers <= 0 || prm->n_heads <= 0 || prm->ffn_hidden <= 0 || prm->vocab_size <= 0 ||
+        prm->max_seq_len <= 0) {
+        return fail(RLH_ERR_INVALID, "rlh_model_create: non-positive dimension");
+    }
+    if (prm->dim % prm->n_heads != 0) return fail(RLH_ERR_INVALID, "rlh_model_create: dim %% n_heads != 0 (transformer.rs:252)");
+    const int hd = prm->dim / prm->n_heads;
+    if (hd != 16 && hd != 32 && hd != 64 && hd != 128) {
+        return fail(RLH_ERR_UNSUPPORTED, "rlh_model_create: head_dim %d (supported: 16, 32, 64, 128)", hd);
+    }
+    if (prm->dim % 8 != 0 || prm->ffn_hidden % 8 != 0) {
+        return fail(RLH_ERR_UNSUPPORTED, "rlh_model_create: dim and ffn_hidden must be multiples of 8 (16-byte weight rows)");
+    }
+    CtxLock lock(ctx);
+    const int wf16 = prm->force_f16 ? 1 : 0;
+    const size_t lds_need = gemv_lds_bytes(prm->ffn_hidden > prm->dim ? prm->ffn_hidden : prm->dim, wf16, wf16);
+    if (lds_need > (size_t)ctx->prop.sharedMemPerBlock && lds_need > 160 * 1024) {
+        return fail(RLH_ERR_UNSUPPORTED, "rlh_model_create: activation vector of %zu bytes does not fit in LDS", lds_need);
+    }
+    rlh_model *m = new rlh_model();
+    m->ctx = ctx;
+    m->prm = *prm;
+    m->prm.percentage_to_gpu = clamp_percentage(prm->percentage_to_gpu);
+    m->head_dim = hd;
+    // transformer.rs:266-268
+    m->last_layer_on_gpu = (int)std::round(m->prm.percentage_to_gpu * (float)(prm->n_layers - 1));
+    m->layers.resize((size_t)prm->n_layers);
+    const int d = prm->dim, F = prm->ffn_hidden, V = prm->vocab_size;
+    int rc = RLH_OK;
+    auto A = [&](Weight &w, int r, int c, int f16) {
+        if (rc == RLH_OK) rc = alloc_weight(w, r, c, f16);
+    };
+    for (auto &L : m->layers) {
+        A(L.wqkv, 3 * d, d, wf16);
+        A(L.wo, d, d, wf16);
+        A(L.w1, F, d, wf16);
+        A(L.w2, d, F, wf16);
+        A(L.w3, F, d, wf16);
+        A(L.attn_norm, 1, d, 0);
+        A(L.ffn_norm, 1, d, 0);
+    }
+    A(m->norm, 1, d, 0);
+    // tok_emb and output are allocated at set_tensor time in the dtype of their source (the reference keeps
+    // both in f32, embedding.rs:41-47 / transformer.rs:302-308; f16 file contents widen exactly).
+    m->tok_emb.rows = V;
+    m->tok_emb.cols = d;
+    m->output.rows = V;
+    m->output.cols = d;
+
+    // RoPE table: compute_freqs_cis (transformer.rs:858-885) in f64, cast to f32 as at its use (:836-837)
+    if (rc == RLH_OK) {
+        std::vector<float2> tab((size_t)prm->max_seq_len * (hd / 2));
+        for (int pos = 0; pos < prm->max_seq_len; pos++) {
+            for (int j = 0; j < hd / 2; j++) {
+                const double freq = 1.0 / std::pow(10000.0, (double)j * 2.0 / (double)hd);
+                const double ang = freq * (double)pos;
+                tab[(size_t)pos * (hd / 2) + j] = make_float2((float)std::cos(ang), (float)std::sin(ang));
+            }
+        }
+        hipError_t e = hipMalloc((void **)&m->freqs, tab.size() * sizeof(float2));
+        if (e == hipSuccess) e = hipMemcpy(m->freqs, tab.data(), tab.size() * sizeof(float2), hipMemcpyHostToDevice);
+        if (e != hipSuccess) rc = fail(RLH_ERR_HIP, "rlh_model_create: RoPE table: %s", hipGetErrorString(e));
+    }
+    auto B = [&](void **p, size_t bytes) {
+        if (rc != RLH_OK) return;
+        hipError_t e = hipMalloc(p, bytes);
+        if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
+        if (e != hipSuccess) rc = fail(e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "rlh_model_create: %s", hipGetErrorString(e));
+    };
+    m->out_cap = prm->max_seq_len + 1;
+    m->prompt_cap = prm->max_seq_len;
+    B((void **)&m->x, sizeof(float) * d);
+    B((void **)&m->q, sizeof(float) * d);
+    B((void **)&m->att, sizeof(float) * d);
+    B((void **)&m->mh, sizeof(float) * F);
+    B((void **)&m->logits, sizeof(float) * V);
+    B((void **)&m->state, sizeof(DecodeState));
+    B((void **)&m->out_tokens, sizeof(int32_t) * m->out_cap);
+    B((void **)&m->prompt_dev, sizeof(int32_t) * m->prompt_cap);
+    B((void **)&m->attn_ws, sizeof(float) * (size_t)prm->n_heads * m->max_splits * (hd + 2));
+    B((void **)&m->attn_counters, sizeof(unsigned int) * prm->n_heads);
+    if (rc == RLH_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(RLH_ERR_HIP, "rlh_model_create: hipDeviceSynchronize failed");
+    if (rc != RLH_OK) {
+        rlh_model_free(m);
+        return rc;
+    }
+    *out = m;
+    return RLH_OK;
+}
+
+extern "C" void rlh_model_free(rlh_model *m) {
+    if (!m) return;
+    CtxLock lock(m->ctx);
+    (void)hipStreamSynchronize(m->ctx->stream);
+    for (auto &L : m->layers) {
+        free_weight(L.wqkv);
+        free_weight(L.wo);
+        free_weight(L.w1);
+        free_weight(L.w2);
+        free_weight(L.w3);
+        free_weight(L.attn_norm);
+        free_weight(L.ffn_norm);
+    }
+    free_weight(m->tok_emb);
+    free_weight(m->norm);
+    free_weight(m->output);
+    void *bufs[] = {m->freqs, m->x, m->q, m->att, m->mh, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws, m->attn_counters};
+    for (void *b : bufs)
+        if (b) (void)hipFree(b);
+    delete m;
+}
+
+struct Slot {
+    Weight *w = nullptr;
+    size_t row_off = 0; // rows into w (fused wqkv)
+    int rows = 0, cols = 0;
+    bool *flag = nullptr;
+};
+
+static int find_slot(rlh_model *m, int kind, int layer, Slot *s) {
+    const int d = m->prm.dim, F = m->prm.ffn_hidden, V = m->prm.vocab_size;
+    if (kind >= RLH_WQ && kind <= RLH_FFN_NORM) {
+        if (layer < 0 || layer >= m->prm.n_layers) return fail(RLH_ERR_INVALID, "layer %d out of range", layer);
+    }
+    Layer *L = (kind >= RLH_WQ && kind <= RLH_FFN_NORM) ? &m->layers[(size_t)layer] : nullptr;
+    switch (kind) {
+    case RLH_TOK_EMB: *s = Slot{&m->tok_emb, 0, V, d, &m->tok_emb.loaded}; break;
+    case RLH_OUTPUT: *s = Slot{&m->output, 0, V, d, &m->output.loaded}; break;
+    case RLH_NORM: *s = Slot{&m->norm, 0, 1, d, &m->norm.loaded}; break;
+    case RLH_WQ: *s = Slot{&L->wqkv, 0, d, d, &L->q_loaded}; break;
+    case RLH_WK: *s = Slot{&L->wqkv, (size_t)d, d, d, &L->k_loaded}; break;
+    case RLH_WV: *s = Slot{&L->wqkv, (size_t)2 * d, d, d, &L->v_loaded}; break;
+    case RLH_WO: *s = Slot{&L->wo, 0, d, d, &L->wo.loaded}; break;
+    case RLH_W1: *s = Slot{&L->w1, 0, F, d, &L->w1.loaded}; break;
+    case RLH_W2: *s = Slot{&L->w2, 0, d, F, &L->w2.loaded}; break;
+    case RLH_W3: *s = Slot{&L->w3, 0, F, d, &L->w3.loaded}; break;
+    case RLH_ATTN_NORM: *s = Slot{&L->attn_norm, 0, 1, d, &L->attn_norm.loaded}; break;
+    case RLH_FFN_NORM: *s = Slot{&L->ffn_norm, 0, 1, d, &L->ffn_norm.loaded}; break;
+    default: return fail(RLH_ERR_INVALID, "unknown tensor kind %d", kind);
+    }
+    return RLH_OK;
+}
+
+extern "C" int rlh_model_set_tensor(rlh_model *m, int kind, int layer, const void *host, int rows, int cols, int src_dtype) {
+    if (!m || !host) return fail(RLH_ERR_INVALID, "rlh_model_set_tensor: NULL argument");
+    if (src_dtype != RLH_F16 && src_dtype != RLH_F32) return fail(RLH_ERR_INVALID, "rlh_model_set_tensor: bad src_dtype %d", src_dtype);
+    CtxLock lock(m->ctx);
+    Slot s;
+    int rc = find_slot(m, kind, layer, &s);
+    if (rc != RLH_OK) return rc;
+    if (rows != s.rows || cols != s.cols) {
+        return fail(RLH_ERR_INVALID, "rlh_model_set_tensor: kind %d expects [%d x %d], got [%d x %d]", kind, s.rows, s.cols, rows, cols);
+    }
+    hipStream_t st = m->ctx->stream;
+    if (kind == RLH_TOK_EMB || kind == RLH_OUTPUT) {
+        // stored in the source's dtype: lossless either way
+        if (s.w->p && s.w->f16 != (src_dtype == RLH_F16)) free_weight(*s.w);
+        if (!s.w->p) {
+            rc = alloc_weight(*s.w, rows, cols, src_dtype == RLH_F16);
+            if (rc != RLH_OK) return rc;
+        }
+    }
+    const size_t n = (size_t)rows * cols;
+    const int dst_f16 = s.w->f16;
+    char *dst = (char *)s.w->p + s.row_off * (size_t)cols * (dst_f16 ? 2 : 4);
+    if ((src_dtype == RLH_F16) == (dst_f16 != 0)) {
+        HIP_TRY(hipMemcpyAsync(dst, host, n * (dst_f16 ? 2 : 4), hipMemcpyHostToDevice, st));
+        HIP_TRY(hipStreamSynchronize(st));
+    } else {
+        // widen (f16 file -> f32 tensor, tensor.rs:2467) or narrow (Tensor::to_f16 under --f16, tensor.rs:2281-2314) on the device
+        void *tmp = nullptr;
+        const size_t sb = n * (src_dtype == RLH_F16 ? 2 : 4);
+        HIP_TRY(hipMalloc(&tmp, sb));
+        hipError_t e = hipMemcpyAsync(tmp, host, sb, hipMemcpyHostToDevice, st);
+        if (e == hipSuccess) e = launch_convert(dst, dst_f16, tmp, src_dtype == RLH_F16, n, st);
+        hipError_t e2 = hipStreamSynchronize(st);
+        (void)hipFree(tmp);
+        HIP_TRY(e);
+        HIP_TRY(e2);
+    }
+    *s.flag = true;
+    return RLH_OK;
+}
+
+extern "C" int rlh_model_get_tensor(rlh_model *m, int kind, int layer, void *host_out, int rows, int cols, int dst_dtype) {
+    if (!m || !host_out) return fail(RLH_ERR_INVALID, "rlh_model_get_tensor: NULL argument");
+    if (dst_dtype != RLH_F16 && dst_dtype != RLH_F32) return fail(RLH_ERR_INVALID, "rlh_model_get_tensor: bad dst_dtype %d", dst_dtype);
+    CtxLock lock(m->ctx);
+    Slot s;
+    int rc = find_slot(m, kind, layer, &s);
+    if (rc != RLH_OK) return rc;
+    if (rows != s.rows || cols != s.cols) return fail(RLH_ERR_INVALID, "rlh_model_get_tensor: shape mismatch");
+    if (!*s.flag || !s.w->p) return fail(RLH_ERR_STATE, "rlh_model_get_tensor: tensor not loaded");
+    const size_t n = (size_t)rows * cols;
+    hipStream_t st = m->ctx->stream;
+    const char *src = (const char *)s.w->p + s.row_off * (size_t)cols * (s.w->f16 ? 2 : 4);
+    const int want_f16 = dst_dtype == RLH_F16;
+    const size_t db = n * (want_f16 ? 2 : 4);
+    if ((s.w->f16 != 0) == (want_f16 != 0)) {
+        HIP_TRY(hipMemcpyAsync(host_out, src, db, hipMemcpyDeviceToHost, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        return RLH_OK;
+    }
+    void *tmp = nullptr;
+    HIP_TRY(hipMalloc(&tmp, db));
+    hipError_t e = launch_convert(tmp, want_f16, src, s.w->f16, n, st);
+    if (e == hipSuccess) e = hipMemcpyAsync(host_out, tmp, db, hipMemcpyDeviceToHost, st);
+    hipError_t e2 = hipStreamSynchronize(st);
+    (void)hipFree(tmp);
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    return RLH_OK;
+}
+
+extern "C" int rlh_model_fill_synthetic(rlh_model *m, uint64_t seed, double std) {
+    if (!m) return fail(RLH_ERR_INVALID, "rlh_model_fill_synthetic: NULL model");
+    CtxLock lock(m->ctx);
+    hipStream_t st = m->ctx->stream;
+    const int d = m->prm.dim;
+    for (Weight *w : {&m->tok_emb, &m->output}) {
+        if (!w->p) {
+            int rc = alloc_weight(*w, w->rows, w->cols, 1);
+            if (rc != RLH_OK) return rc;
+        }
+    }
+    auto fill = [&](Weight &w, size_t row_off, int rows, int kind, int layer) -> hipError_t {
+        char *dst = (char *)w.p + row_off * (size_t)w.cols * (w.f16 ? 2 : 4);
+        return launch_synth_fill(dst, w.f16, (uint64_t)rows * w.cols, synth_key(seed, SYNTH_STREAM_TENSOR(kind, layer)), std, st);
+    };
+    HIP_TRY(fill(m->tok_emb, 0, m->tok_emb.rows, RLH_TOK_EMB, 0));
+    HIP_TRY(fill(m->output, 0, m->output.rows, RLH_OUTPUT, 0));
+    HIP_TRY(launch_fill_f32((float *)m->norm.p, (uint64_t)d, 1.0f, st));
+    m->tok_emb.loaded = m->output.loaded = m->norm.loaded = true;
+    for (int l = 0; l < m->prm.n_layers; l++) {
+        Layer &L = m->layers[(size_t)l];
+        HIP_TRY(fill(L.wqkv, 0, d, RLH_WQ, l));
+        HIP_TRY(fill(L.wqkv, (size_t)d, d, RLH_WK, l));
+        HIP_TRY(fill(L.wqkv, (size_t)2 * d, d, RLH_WV, l));
+        HIP_TRY(fill(L.wo, 0, L.wo.rows, RLH_WO, l));
+        HIP_TRY(fill(L.w1, 0, L.w1.rows, RLH_W1, l));
+        HIP_TRY(fill(L.w2, 0, L.w2.rows, RLH_W2, l));
+        HIP_TRY(fill(L.w3, 0, L.w3.rows, RLH_W3, l));
+        HIP_TRY(launch_fill_f32((float *)L.attn_norm.p, (uint64_t)d, 1.0f, st));
+        HIP_TRY(launch_fill_f32((float *)L.ffn_norm.p, (uint64_t)d, 1.0f, st));
+        L.q_loaded = L.k_loaded = L.v_loaded = true;
+        L.wo.loaded = L.w1.loaded = L.w2.loaded = L.w3.loaded = L.attn_norm.loaded = L.ffn_norm.loaded = true;
+    }
+    HIP_TRY(hipStreamSynchronize(st));
+    return RLH_OK;
+}
+
+extern "C" int rlh_model_layers_on_gpu(const rlh_model *m, int *last_layer_on_gpu) {
+    if (!m || !last_layer_on_gpu) return fail(RLH_ERR_INVALID, "rlh_model_layers_on_gpu: NULL argument");
+    *last_layer_on_gpu = m->last_layer_on_gpu;
+    return RLH_OK;
+}
+
+extern "C" int rlh_model_decode_bytes(const rlh_model *m, int T, uint64_t *bytes) {
+    if (!m || !bytes || T < 1) return fail(RLH_ERR_INVALID, "rlh_model_decode_bytes: bad argument");
+    const uint64_t d = (uint64_t)m->prm.dim, F = (uint64_t)m->prm.ffn_hidden, V = (uint64_t)m->prm.vocab_size, L = (uint64_t)m->prm.n_layers;
+    const uint64_t es = m->prm.force_f16 ? 2 : 4;
+    const uint64_t head_es = (m->output.p && !m->output.f16) ? 4 : 2;
+    uint64_t b = L * (4 * d * d + 3 * d * F) * es + V * d * head_es;
+    b += L * 2 * (uint64_t)T * d * es; // K and V rows read
+    b += L * 2 * d * es;               // K and V row written
+    *bytes = b;
+    return RLH_OK;
+}
+
+static int model_ready(const rlh_model *m) {
+    if (!m->tok_emb.loaded || !m->output.loaded || !m->norm.loaded) return 0;
+    for (const auto &L : m->layers) {
+        if (!(L.q_loaded && L.k_loaded && L.v_loaded && L.wo.loaded && L.w1.loaded && L.w2.loaded && L.w3.loaded && L.attn_norm.loaded &&
+              L.ffn_norm.loaded))
+            return 0;
+    }
+    return 1;
+}
+
+// ------------------------------------------------------------------------------------------------
+// caches
+// ------------------------------------------------------------------------------------------------
+extern "C" int rlh_caches_create(rlh_model *m, rlh_caches **out) {
+    if (!m || !out) return fail(RLH_ERR_INVALID, "rlh_caches_create: NULL argument");
+    *out = nullptr;
+    CtxLock lock(m->ctx);
+    rlh_caches *c = new rlh_caches();
+    c->model = m;
+    c->f16 = m->prm.force_f16 ? 1 : 0; // transformer.rs:138-142
+    c->bytes_each = (size_t)m->prm.n_layers * m->prm.n_heads * m->prm.max_seq_len * m->head_dim * (c->f16 ? 2 : 4);
+    hipError_t e = hipMalloc(&c->k, c->bytes_each);
+    if (e == hipSuccess) e = hipMalloc(&c->v, c->bytes_each);
+    if (e == hipSuccess) e = hipMemsetAsync(c->k, 0, c->bytes_each, m->ctx->stream); // Tensor::zeros
+    if (e == hipSuccess) e = hipMemsetAsync(c->v, 0, c->bytes_each, m->ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(m->ctx->stream);
+    if (e != hipSuccess) {
+        if (c->k) (void)hipFree(c->k);
+        if (c->v) (void)hipFree(c->v);
+        delete c;
+        return fail(e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "rlh_caches_create: %s", hipGetErrorString(e));
+    }
+    *out = c;
+    return RLH_OK;
+}
+
+extern "C" int rlh_caches_true_clone(const rlh_caches *src, rlh_caches **out) {
+    if (!src || !out) return fail(RLH_ERR_INVALID, "rlh_caches_true_clone: NULL argument");
+    *out = nullptr;
+    rlh_ctx *ctx = src->model->ctx;
+    CtxLock lock(ctx);
+    rlh_caches *c = new rlh_caches(*src);
+    c->k = c->v = nullptr;
+    hipError_t e = hipMalloc(&c->k, c->bytes_each);
+    if (e == hipSuccess) e = hipMalloc(&c->v, c->bytes_each);
+    if (e == hipSuccess) e = hipMemcpyAsync(c->k, src->k, c->bytes_each, hipMemcpyDeviceToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(c->v, src->v, c->bytes_each, hipMemcpyDeviceToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        if (c->k) (void)hipFree(c->k);
+        if (c->v) (void)hipFree(c->v);
+        delete c;
+        return fail(e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "rlh_caches_true_clone: %s", hipGetErrorString(e));
+    }
+    *out = c;
+    return RLH_OK;
+}
+
+extern "C" int rlh_caches_shift_left(rlh_caches *c, int shifts) {
+    if (!c || shifts < 0) return fail(RLH_ERR_INVALID, "rlh_caches_shift_left: bad argument");
+    if (shifts == 0) return RLH_OK;
+    rlh_model *m = c->model;
+    CtxLock lock(m->ctx);
+    const size_t planes = (size_t)m->prm.n_layers * m->prm.n_heads;
+    HIP_TRY(launch_cache_shift_left(c->k, c->f16, planes, m->prm.max_seq_len, m->head_dim, shifts, m->ctx->stream));
+    HIP_TRY(launch_cache_shift_left(c->v, c->f16, planes, m->prm.max_seq_len, m->head_dim, shifts, m->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" void rlh_caches_free(rlh_caches *c) {
+    if (!c) return;
+    CtxLock lock(c->model->ctx);
+    (void)hipStreamSynchronize(c->model->ctx->stream);
+    if (c->k) (void)hipFree(c->k);
+    if (c->v) (void)hipFree(c->v);
+    delete c;
+}
+
+extern "C" int rlh_caches_read(const rlh_caches *c, int layer, int head, int which, float *host_out) {
+    if (!c || !host_out) return fail(RLH_ERR_INVALID, "rlh_caches_read: NULL argument");
+    rlh_model *m = c->model;
+    if (layer < 0 || layer >= m->prm.n_layers || head < 0 || head >= m->prm.n_heads) return fail(RLH_ERR_INVALID, "rlh_caches_read: index out of range");
+    CtxLock lock(m->ctx);
+    const size_t per_plane = (size_t)m->prm.max_seq_len * m->head_dim;
+    const size_t off = ((size_t)layer * m->prm.n_heads + head) * per_plane * (c->f16 ? 2 : 4);
+    const char *plane = (const char *)(which ? c->v : c->k) + off;
+    float *tmp = nullptr;
+    HIP_TRY(hipMalloc((void **)&tmp, per_plane * 4));
+    hipError_t e = launch_cache_read(tmp, plane, c->f16, m->prm.max_seq_len, m->head_dim, m->ctx->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(host_out, tmp, per_plane * 4, hipMemcpyDeviceToHost, m->ctx->stream);
+    hipError_t e2 = hipStreamSynchronize(m->ctx->stream);
+    (void)hipFree(tmp);
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    return RLH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// forward
+// ------------------------------------------------------------------------------------------------
+static void attn_config(const rlh_model *m, int T, int *splits, int *chunk_cap) {
+    // One block per (head, split).  Aim for chunks of >= 64 positions and at most max_splits splits.
+    int S = (T + 63) / 64;
+    if (S < 1) S = 1;
+    if (S > m->max_splits) S = m->max_splits;
+    int chunk = (T + S - 1) / S;
+    chunk = (chunk + 15) & ~15;
+    *splits = S;
+    *chunk_cap = chunk;
+}
+
+enum StepKernel { kStepQkv = 0, kStepAttn = 1, kStepWo = 2, kStepW13 = 3, kStepW2 = 4, kStepHead = 5 };
+
+// Enqueues one of the five kernels of layer l (or the output head) for the token described by the device
+// state.  T_host = position + 1 as known to the host (sizes the attention grid).
+static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, int T_host) {
+    hipStream_t st = m->ctx->stream;
+    const rlh_model_params &P = m->prm;
+    const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size;
+    const int f16 = P.force_f16 ? 1 : 0;
+    const float eps = (float)P.norm_eps; // add_scalar(self.eps as f32), transformer.rs:477
+    GemvParams g{};
+    g.stream_weights = m->stream_weights;
+    g.w_is_f16 = f16;
+    g.x_f16 = f16;
+    g.round_y = f16;
+    g.eps = eps;
+    if (which == kStepHead) {
+        // final norm + output head: f32 activations, no rounding (transformer.rs:378-381; tensor.rs:1837-1918)
+        GemvParams p{};
+        p.stream_weights = m->stream_weights;
+        p.w = m->output.p;
+        p.w_is_f16 = m->output.f16;
+        p.x = m->x;
+        p.x_f16 = 0;
+        p.round_y = 0;
+        p.norm_w = (const float *)m->norm.p;
+        p.eps = eps;
+        p.y = m->logits;
+        p.n_rows = V;
+        p.k = d;
+        HIP_TRY(launch_gemv(p, kEpiStore, st));
+        return RLH_OK;
+    }
+    Layer &L = m->layers[(size_t)l];
+    const size_t layer_elems = (size_t)P.n_heads * P.max_seq_len * m->head_dim;
+    const size_t ces = c->f16 ? 2 : 4;
+    void *ck = (char *)c->k + (size_t)l * layer_elems * ces;
+    void *cv = (char *)c->v + (size_t)l * layer_elems * ces;
+    switch (which) {
+    case kStepQkv: {
+        // attention_norm + wq|wk|wv + RoPE + cache write (transformer.rs:432, 665-668, 694-725, 751-761)
+        GemvParams p = g;
+        p.w = L.wqkv.p;
+        p.x = m->x;
+        p.norm_w = (const float *)L.attn_norm.p;
+        p.y = m->q;
+        p.n_rows = 3 * d;
+        p.k = d;
+        p.state = m->state;
+        p.freqs = m->freqs;
+        p.cache_k = ck;
+        p.cache_v = cv;
+        p.cache_f16 = c->f16;
+        p.dim = d;
+        p.head_dim = m->head_dim;
+        p.max_seq_len = P.max_seq_len;
+        HIP_TRY(launch_gemv(p, kEpiRopeKv, st));
+        break;
+    }
+    case kStepAttn: {
+        // scores, softmax, P.V (transformer.rs:762-779) + f16 rounding point before wo (:793-796)
+        int splits, chunk_cap;
+        attn_config(m, T_host, &splits, &chunk_cap);
+        AttnDecodeParams a{};
+        a.q = m->q;
+        a.cache_k = ck;
+        a.cache_v = cv;
+        a.cache_f16 = c->f16;
+        a.state = m->state;
+        a.n_heads = P.n_heads;
+        a.head_dim = m->head_dim;
+        a.max_seq_len = P.max_seq_len;
+        a.n_splits = splits;
+        a.chunk_cap = chunk_cap;
+        a.out = m->att;
+        a.round_out = f16;
+        a.workspace = m->attn_ws;
+        a.counters = m->attn_counters;
+        HIP_TRY(launch_attn_decode(a, st));
+        break;
+    }
+    case kStepWo: {
+        // wo + residual (transformer.rs:783-819, 442)
+        GemvParams p = g;
+        p.w = L.wo.p;
+        p.x = m->att;
+        p.y = m->x;
+        p.n_rows = d;
+        p.k = d;
+        HIP_TRY(launch_gemv(p, kEpiResAdd, st));
+        break;
+    }
+    case kStepW13: {
+        // ffn_norm + w1|w3 + SiLU * gate (transformer.rs:443, 537-565)
+        GemvParams p = g;
+        p.w = L.w1.p;
+        p.w_b = L.w3.p;
+        p.x = m->x;
+        p.norm_w = (const float *)L.ffn_norm.p;
+        p.y = m->mh;
+        p.n_rows = F;
+        p.k = d;
+        HIP_TRY(launch_gemv(p, kEpiSilu, st));
+        break;
+    }
+    case kStepW2: {
+        // w2 + residual (transformer.rs:568-570, 445)
+        GemvParams p = g;
+        p.w = L.w2.p;
+        p.x = m->mh;
+        p.y = m->x;
+        p.n_rows = d;
+        p.k = F;
+        HIP_TRY(launch_gemv(p, kEpiResAdd, st));
+        break;
+    }
+    default: return fail(RLH_ERR_INVALID, "unknown step kernel %d", which);
+    }
+    return RLH_OK;
+}
+
+// Enqueues one token step (the body of Transformer::forward for a single row, transformer.rs:361-381):
+// reads state->token / state->pos on the device.
+static int enqueue_token_step(rlh_model *m, rlh_caches *c, int T_host, bool with_head) {
+    HIP_TRY(launch_embed(m->tok_emb.p, m->tok_emb.f16, m->prm.dim, m->state, m->x, m->ctx->stream));
+    for (int l = 0; l < m->prm.n_layers; l++) {
+        for (int which = kStepQkv; which <= kStepW2; which++) {
+            int rc = enqueue_step_kernel(m, c, l, which, T_host);
+            if (rc != RLH_OK) return rc;
+        }
+    }
+    if (with_head) return enqueue_step_kernel(m, c, 0, kStepHead, T_host);
+    return RLH_OK;
+}
+
+static int check_forward_args(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, const char *who) {
+    if (!m || !c || !tokens) return fail(RLH_ERR_INVALID, "%s: NULL argument", who);
+    if (c->model != m) return fail(RLH_ERR_STATE, "%s: caches belong to another model", who);
+    if (!model_ready(m)) return fail(RLH_ERR_STATE, "%s: model has tensors that were never set", who);
+    if (n < 1) return fail(RLH_ERR_INVALID, "%s: n must be >= 1", who);
+    if (n > 1 && start_pos != 0) {
+        return fail(RLH_ERR_INVALID, "%s: n > 1 needs start_pos == 0 (the reference's mask is n x n, transformer.rs:350-357)", who);
+    }
+    if (start_pos < 0 || start_pos + n > m->prm.max_seq_len) {
+        return fail(RLH_ERR_STATE, "%s: start_pos + n = %d exceeds max_seq_len %d", who, start_pos + n, m->prm.max_seq_len);
+    }
+    for (int i = 0; i < n; i++) {
+        if (tokens[i] < 0 || tokens[i] >= m->prm.vocab_size) return fail(RLH_ERR_INVALID, "%s: token id %d out of range", who, tokens[i]);
+    }
+    return RLH_OK;
+}
+
+// Runs the n tokens of one forward call; logits of the last one are left in m->logits.
+static int enqueue_forward(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos) {
+    hipStream_t st = m->ctx->stream;
+    m->next_pos = -1;
+    m->greedy_caches = nullptr;
+    HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
+    HIP_TRY(launch_set_state(m->state, start_pos, tokens[0], 1, st));
+    for (int i = 0; i < n; i++) {
+        int rc = enqueue_token_step(m, c, start_pos + i + 1, i == n - 1);
+        if (rc != RLH_OK) return rc;
+        if (i + 1 < n) HIP_TRY(launch_advance_pos(m->state, m->prompt_dev, i + 1, st));
+    }
+    return RLH_OK;
+}
+
+extern "C" int rlh_forward(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, float *logits_out) {
+    int rc = check_forward_args(m, c, tokens, n, start_pos, "rlh_forward");
+    if (rc != RLH_OK) return rc;
+    if (!logits_out) return fail(RLH_ERR_INVALID, "rlh_forward: logits_out is NULL");
+    CtxLock lock(m->ctx);
+    rc = enqueue_forward(m, c, tokens, n, start_pos);
+    if (rc != RLH_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(logits_out, m->logits, sizeof(float) * (size_t)m->prm.vocab_size, hipMemcpyDeviceToHost, m->ctx->stream));
+    HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, int32_t *next_token) {
+    int rc = check_forward_args(m, c, tokens, n, start_pos, "rlh_forward_greedy");
+    if (rc != RLH_OK) return rc;
+    if (!next_token) return fail(RLH_ERR_INVALID, "rlh_forward_greedy: next_token is NULL");
+    CtxLock lock(m->ctx);
+    hipStream_t st = m->ctx->stream;
+    rc = enqueue_forward(m, c, tokens, n, start_pos);
+    if (rc != RLH_OK) return rc;
+    HIP_TRY(launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st));
+    HIP_TRY(hipMemcpyAsync(next_token, m->out_tokens, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    m->next_pos = start_pos + n;
+    m->greedy_caches = c;
+    return RLH_OK;
+}
+
+extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *prompt, int n_prompt, int n_new, int32_t *out_tokens,
+                                   float *ms_first, float *ms_per_token) {
+    int rc = check_forward_args(m, c, prompt, n_prompt, 0, "rlh_generate_greedy");
+    if (rc != RLH_OK) return rc;
+    if (!out_tokens || n_new < 1) return fail(RLH_ERR_INVALID, "rlh_generate_greedy: bad output arguments");
+    if (n_prompt + n_new - 1 > m->prm.max_seq_len) {
+        return fail(RLH_ERR_STATE, "rlh_generate_greedy: %d prompt + %d new tokens exceed max_seq_len %d", n_prompt, n_new, m->prm.max_seq_len);
+    }
+    CtxLock lock(m->ctx);
+    hipStream_t st = m->ctx->stream;
+    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    HIP_TRY(hipEventCreate(&e2));
+    auto cleanup = [&]() {
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        (void)hipEventDestroy(e2);
+    };
+    hipError_t e = hipEventRecord(e0, st);
+    if (e == hipSuccess) {
+        rc = enqueue_forward(m, c, prompt, n_prompt, 0);
+        if (rc == RLH_OK) e = launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st);
+    }
+    if (rc == RLH_OK && e == hipSuccess) e = hipEventRecord(e1, st);
+    for (int i = 1; rc == RLH_OK && e == hipSuccess && i < n_new; i++) {
+        // the new token sits at position n_prompt + i - 1; attention spans n_prompt + i positions
+        rc = enqueue_token_step(m, c, n_prompt + i, true);
+        if (rc == RLH_OK) e = launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st);
+    }
+    if (rc == RLH_OK && e == hipSuccess) e = hipEventRecord(e2, st);
+    if (rc == RLH_OK && e == hipSuccess) e = hipMemcpyAsync(out_tokens, m->out_tokens, sizeof(int32_t) * (size_t)n_new, hipMemcpyDeviceToHost, st);
+    if (rc == RLH_OK && e == hipSuccess) e = hipStreamSynchronize(st);
+    if (rc == RLH_OK && e == hipSuccess) {
+        float a = 0.0f, b = 0.0f;
+        (void)hipEventElapsedTime(&a, e0, e1);
+        (void)hipEventElapsedTime(&b, e1, e2);
+        if (ms_first) *ms_first = a;
+        if (ms_per_token) *ms_per_token = n_new > 1 ? b / (float)(n_new - 1) : 0.0f;
+    }
+    cleanup();
+    if (rc != RLH_OK) return rc;
+    HIP_TRY(e);
+    m->next_pos = n_prompt + n_new - 1;
+    m->greedy_caches = c;
+    return RLH_OK;
+}
+
+extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32_t *out_tokens, float *ms_total) {
+    if (!m || !c || !out_tokens || n_steps < 1) return fail(RLH_ERR_INVALID, "rlh_decode_greedy: bad argument");
+    if (c->model != m) return fail(RLH_ERR_STATE, "rlh_decode_greedy: caches belong to another model");
+    if (m->next_pos < 0 || m->greedy_caches != c) {
+        return fail(RLH_ERR_STATE, "rlh_decode_greedy: no sampled token on the device for these caches (call rlh_forward_greedy or rlh_generate_greedy first)");
+    }
+    if (m->next_pos + n_steps > m->prm.max_seq_len) {
+        return fail(RLH_ERR_STATE, "rlh_decode_greedy: position %d + %d steps exceed max_seq_len %d", m->next_pos, n_steps, m->prm.max_seq_len);
+    }
+    if (n_steps > m->out_cap) return fail(RLH_ERR_INVALID, "rlh_decode_greedy: n_steps too large");
+    CtxLock lock(m->ctx);
+    hipStream_t st = m->ctx->stream;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    HIP_TRY(hipEventCreate(&e0));
+    hipError_t e = hipEventCreate(&e1);
+    int rc = RLH_OK;
+    // keep pos/token, restart the output list
+    if (e == hipSuccess) e = launch_reset_out(m->state, st);
+    if (e == hipSuccess) e = hipEventRecord(e0, st);
+    for (int i = 0; rc == RLH_OK && e == hipSuccess && i < n_steps; i++) {
+        rc = enqueue_token_step(m, c, m->next_pos + i + 1, true);
+        if (rc == RLH_OK) e = launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st);
+    }
+    if (rc == RLH_OK && e == hipSuccess) e = hipEventRecord(e1, st);
+    if (rc == RLH_OK && e == hipSuccess) e = hipMemcpyAsync(out_tokens, m->out_tokens, sizeof(int32_t) * (size_t)n_steps, hipMemcpyDeviceToHost, st);
+    hipError_t e2 = hipStreamSynchronize(st);
+    float ms = 0.0f;
+    if (rc == RLH_OK && e == hipSuccess && e2 == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (rc != RLH_OK || e != hipSuccess || e2 != hipSuccess) m->next_pos = -1;
+    if (rc != RLH_OK) return rc;
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    if (ms_total) *ms_total = ms;
+    m->next_pos += n_steps;
+    return RLH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// measurement aids
+// ------------------------------------------------------------------------------------------------
+extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int T, int iters, float *us_per_launch, uint64_t *bytes_per_launch) {
+    if (!m || !c || !us_per_launch || iters < 1) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad argument");
+    if (c->model != m) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: caches belong to another model");
+    if (!model_ready(m)) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: model has tensors that were never set");
+    if (T < 1 || T > m->prm.max_seq_len || which < kStepQkv || which > kStepHead) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad T or kernel id");
+    CtxLock lock(m->ctx);
+    hipStream_t st = m->ctx->stream;
+    const uint64_t d = (uint64_t)m->prm.dim, F = (uint64_t)m->prm.ffn_hidden, V = (uint64_t)m->prm.vocab_size;
+    const uint64_t es = m->prm.force_f16 ? 2 : 4;
+    if (bytes_per_launch) {
+        // algorithmic bytes: the weights the kernel must read once + its input and output vectors
+        switch (which) {
+        case kStepQkv: *bytes_per_launch = 3 * d * d * es + d * 4 + d * 4 + d * 4 + 2 * d * es; break;
+        case kStepAttn: *bytes_per_launch = 2 * (uint64_t)T * d * es + d * 4 + d * 4; break;
+        case kStepWo: *bytes_per_launch = d * d * es + d * 4 + 2 * d * 4; break;
+        case kStepW13: *bytes_per_launch = 2 * F * d * es + d * 4 + d * 4 + F * 4; break;
+        case kStepW2: *bytes_per_launch = d * F * es + F * 4 + 2 * d * 4; break;
+        default: *bytes_per_launch = V * d * (m->output.f16 ? 2 : 4) + d * 4 + d * 4 + V * 4; break;
+        }
+    }
+    HIP_TRY(launch_set_state(m->state, T - 1, 3 % m->prm.vocab_size, 1, st));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    int rc = RLH_OK;
+    const int L = m->prm.n_layers;
+    for (int i = 0; rc == RLH_OK && i < (L < 4 ? L : 4); i++) rc = enqueue_step_kernel(m, c, i % L, which, T); // warm-up
+    hipError_t e = hipEventRecord(e0, st);
+    for (int i = 0; rc == RLH_OK && e == hipSuccess && i < iters; i++) rc = enqueue_step_kernel(m, c, i % L, which, T);
+    if (e == hipSuccess) e = hipEventRecord(e1, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != RLH_OK) return rc;
+    HIP_TRY(e);
+    *us_per_launch = ms * 1000.0f / (float)iters;
+    return RLH_OK;
+}
+
+extern "C" int rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int round_x, int round_y, int n_buffers, int iters, float *us_per_launch) {
+    if (!ctx || !us_per_launch || rows < 1 || k < 1 || n_buffers < 1 || iters < 1) return fail(RLH_ERR_INVALID, "rlh_time_gemv: bad argument");
+    const int f16 = w_dtype == RLH_F16;
+    if (k % (f16 ? 8 : 4) != 0) return fail(RLH_ERR_UNSUPPORTED, "rlh_time_gemv: k must be a multiple of %d", f16 ? 8 : 4);
+    CtxLock lock(ctx);
+    hipStream_t st = ctx->stream;
+    const size_t wbytes = (size_t)rows * k * (f16 ? 2 : 4);
+    std::vector<void *> bufs((size_t)n_buffers, nullptr);
+    float *x = nullptr, *y = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipSuccess;
+    for (int i = 0; e == hipSuccess && i < n_buffers; i++) {
+        e = hipMalloc(&bufs[(size_t)i], wbytes);
+        if (e == hipSuccess) e = launch_synth_fill(bufs[(size_t)i], f16, (uint64_t)rows * k, synth_key(99, (uint64_t)i), 0.02, st);
+    }
+    if (e == hipSuccess) e = hipMalloc((void **)&x, sizeof(float) * (size_t)k);
+    if (e == hipSuccess) e = hipMalloc((void **)&y, sizeof(float) * (size_t)rows);
+    if (e == hipSuccess) e = launch_fill_f32(x, (uint64_t)k, 0.5f, st);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    GemvParams p{};
+    p.w_is_f16 = f16;
+    p.x = x;
+    p.x_f16 = round_x ? 1 : 0;
+    p.round_y = round_y ? 1 : 0;
+    p.y = y;
+    p.n_rows = rows;
+    p.k = k;
+    p.stream_weights = 1;
+    for (int i = 0; e == hipSuccess && i < n_buffers; i++) {
+        p.w = bufs[(size_t)i];
+        e = launch_gemv(p, kEpiStore, st);
+    }
+    if (e == hipSuccess) e = hipEventRecord(e0, st);
+    for (int i = 0; e == hipSuccess && i < iters; i++) {
+        p.w = bufs[(size_t)(i % n_buffers)];
+        e = launch_gemv(p, kEpiStore, st);
+    }
+    if (e == hipSuccess) e = hipEventRecord(e1, st);
+    hipError_t e2 = hipStreamSynchronize(st);
+    float ms = 0.0f;
+    if (e == hipSuccess && e2 == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    for (void *b : bufs)
+        if (b) (void)hipFree(b);
+    if (x) (void)hipFree(x);
+    if (y) (void)hipFree(y);
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    *us_per_launch = ms * 1000.0f / (float)iters;
+    return RLH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// op level
+// ------------------------------------------------------------------------------------------------
+extern "C" int rlh_tensor_alloc(rlh_ctx *ctx, int rows, int cols, int dtype, rlh_tensor **out) {
+    if (!ctx || !out || rows <= 0 || cols <= 0 || (dtype != RLH_F16 && dtype != RLH_F32)) return fail(RLH_ERR_INVALID, "rlh_tensor_alloc: bad argument");
+    *out = nullptr;
+    CtxLock lock(ctx);
+    rlh_tensor *t = new rlh_tensor();
+    t->ctx = ctx;
+    t->rows = rows;
+    t->cols = cols;
+    t->dtype = dtype;
+    hipError_t e = hipMalloc(&t->p, t->count() * t->esize());
+    if (e == hipSuccess) e = hipMemsetAsync(t->p, 0, t->count() * t->esize(), ctx->stream);
+    if (e != hipSuccess) {
+        if (t->p) (void)hipFree(t->p);
+        delete t;
+        return fail(e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "rlh_tensor_alloc: %s", hipGetErrorString(e));
+    }
+    *out = t;
+    return RLH_OK;
+}
+
+extern "C" int rlh_tensor_upload(rlh_ctx *ctx, const void *host, int rows, int cols, int cols_capacity, int dtype, rlh_tensor **out) {
+    if (!host || cols_capacity < cols) return fail(RLH_ERR_INVALID, "rlh_tensor_upload: bad argument");
+    int rc = rlh_tensor_alloc(ctx, rows, cols, dtype, out);
+    if (rc != RLH_OK) return rc;
+    CtxLock lock(ctx);
+    rlh_tensor *t = *out;
+    const size_t es = t->esize();
+    hipError_t e = hipMemcpy2DAsync(t->p, (size_t)cols * es, host, (size_t)cols_capacity * es, (size_t)cols * es, (size_t)rows,
+                                    hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream); // the host buffer is the caller's again on return
+    if (e != hipSuccess) {
+        rlh_tensor_free(t);
+        *out = nullptr;
+        return fail(RLH_ERR_HIP, "rlh_tensor_upload: %s", hipGetErrorString(e));
+    }
+    return RLH_OK;
+}
+
+extern "C" int rlh_tensor_download(rlh_tensor *t, void *host, int cols_capacity, rlh_event **ev) {
+    if (!t || !host || cols_capacity < t->cols) return fail(RLH_ERR_INVALID, "rlh_tensor_download: bad argument");
+    CtxLock lock(t->ctx);
+    const size_t es = t->esize();
+    HIP_TRY(hipMemcpy2DAsync(host, (size_t)cols_capacity * es, t->p, (size_t)t->cols * es, (size_t)t->cols * es, (size_t)t->rows,
+                             hipMemcpyDeviceToHost, t->ctx->stream));
+    if (ev) {
+        int rc = rlh_event_record(t->ctx, ev);
+        if (rc != RLH_OK) return rc;
+    } else {
+        HIP_TRY(hipStreamSynchronize(t->ctx->stream));
+    }
+    return RLH_OK;
+}
+
+extern "C" void rlh_tensor_free(rlh_tensor *t) {
+    if (!t) return;
+    CtxLock lock(t->ctx);
+    (void)hipStreamSynchronize(t->ctx->stream);
+    if (t->p) (void)hipFree(t->p);
+    delete t;
+}
+
+extern "C" int rlh_tensor_shape(const rlh_tensor *t, int *rows, int *cols, int *dtype) {
+    if (!t) return fail(RLH_ERR_INVALID, "rlh_tensor_shape: NULL tensor");
+    if (rows) *rows = t->rows;
+    if (cols) *cols = t->cols;
+    if (dtype) *dtype = t->dtype;
+    return RLH_OK;
+}
+
+extern "C" int rlh_event_record(rlh_ctx *ctx, rlh_event **out) {
+    if (!ctx || !out) return fail(RLH_ERR_INVALID, "rlh_event_record: NULL argument");
+    CtxLock lock(ctx);
+    rlh_event *ev = new rlh_event();
+    ev->ctx = ctx;
+    hipError_t e = hipEventCreate(&ev->ev);
+    if (e == hipSuccess) e = hipEventRecord(ev->ev, ctx->stream);
+    if (e != hipSuccess) {
+        if (ev->ev) (void)hipEventDestroy(ev->ev);
+        delete ev;
+        return fail(RLH_ERR_HIP, "rlh_event_record: %s", hipGetErrorString(e));
+    }
+    *out = ev;
+    return RLH_OK;
+}
+
+extern "C" int rlh_event_wait(rlh_event *ev) {
+    if (!ev) return fail(RLH_ERR_INVALID, "rlh_event_wait: NULL event");
+    hipError_t e = hipEventSynchronize(ev->ev);
+    (void)hipEventDestroy(ev->ev);
+    delete ev;
+    if (e != hipSuccess) return fail(RLH_ERR_HIP, "rlh_event_wait: %s", hipGetErrorString(e));
+    return RLH_OK;
+}
+
+extern "C" int rlh_event_elapsed_ms(rlh_event *start, rlh_event *stop, float *ms) {
+    if (!start || !stop || !ms) return fail(RLH_ERR_INVALID, "rlh_event_elapsed_ms: NULL argument");
+    HIP_TRY(hipEventSynchronize(stop->ev));
+    HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
+    return RLH_OK;
+}
+
+extern "C" void rlh_event_free(rlh_event *ev) {
+    if (!ev) return;
+    if (ev->ev) (void)hipEventDestroy(ev->ev);
+    delete ev;
+}
+
+static int same_shape(const rlh_tensor *a, const rlh_tensor *b) { return a->rows == b->rows && a->cols == b->cols && a->dtype == b->dtype; }
+
+extern "C" int rlh_copy_inplace(rlh_tensor *dst, const rlh_tensor *src) {
+    if (!dst || !src || !same_shape(dst, src)) return fail(RLH_ERR_INVALID, "rlh_copy_inplace: shape/dtype mismatch");
+    CtxLock lock(dst->ctx);
+    HIP_TRY(hipMemcpyAsync(dst->p, src->p, dst->count() * dst->esize(), hipMemcpyDeviceToDevice, dst->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_transpose_from(rlh_tensor *dst, const rlh_tensor *src) {
+    if (!dst || !src || dst->rows != src->cols || dst->cols != src->rows || dst->dtype != src->dtype) {
+        return fail(RLH_ERR_INVALID, "rlh_transpose_from: shape/dtype mismatch");
+    }
+    CtxLock lock(dst->ctx);
+    HIP_TRY(launch_transpose(dst->p, src->p, src->rows, src->cols, src->dtype == RLH_F16, dst->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_hadamard_product_inplace(rlh_tensor *dst, const rlh_tensor *src) {
+    if (!dst || !src || !same_shape(dst, src)) return fail(RLH_ERR_INVALID, "rlh_hadamard_product_inplace: shape/dtype mismatch");
+    CtxLock lock(dst->ctx);
+    HIP_TRY(launch_hadamard(dst->p, src->p, dst->count(), dst->dtype == RLH_F16, dst->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_silu_inplace(rlh_tensor *t) {
+    if (!t) return fail(RLH_ERR_INVALID, "rlh_silu_inplace: NULL tensor");
+    CtxLock lock(t->ctx);
+    HIP_TRY(launch_silu(t->p, t->count(), t->dtype == RLH_F16, t->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_gemv(rlh_tensor *y, const rlh_tensor *w, const rlh_tensor *x, int round_x, int round_y) {
+    if (!y || !w || !x) return fail(RLH_ERR_INVALID, "rlh_gemv: NULL argument");
+    if (x->dtype != RLH_F32 || y->dtype != RLH_F32) return fail(RLH_ERR_INVALID, "rlh_gemv: x and y must be f32");
+    if (x->rows != 1 || y->rows != 1 || x->cols != w->cols || y->cols != w->rows) return fail(RLH_ERR_INVALID, "rlh_gemv: shape mismatch");
+    const int vec = w->dtype == RLH_F16 ? 8 : 4;
+    if (w->cols % vec != 0) return fail(RLH_ERR_UNSUPPORTED, "rlh_gemv: k must be a multiple of %d", vec);
+    CtxLock lock(y->ctx);
+    GemvParams p{};
+    p.w = w->p;
+    p.w_is_f16 = w->dtype == RLH_F16;
+    p.x = (const float *)x->p;
+    p.x_f16 = round_x ? 1 : 0;
+    p.round_y = round_y ? 1 : 0;
+    p.y = (float *)y->p;
+    p.n_rows = w->rows;
+    p.k = w->cols;
+    p.stream_weights = 1;
+    HIP_TRY(launch_gemv(p, kEpiStore, y->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tensor *src, const rlh_tensor *other) {
+    if (!dst || !src || !other) return fail(RLH_ERR_INVALID, "rlh_matrix_mul_inplace_transposed: NULL argument");
+    if (src->cols != other->cols) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication %dx%d vs %dx%d", src->rows, src->cols, other->rows, other->cols);
+    if (src->dtype != other->dtype || dst->dtype != src->dtype) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication, different dtypes");
+    if (dst->rows != src->rows) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication, different number of rows");
+    if (dst->cols != other->rows) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication, different number of cols");
+    const int f16 = src->dtype == RLH_F16;
+    if (src->cols % (f16 ? 8 : 4) != 0) return fail(RLH_ERR_UNSUPPORTED, "rlh_matrix_mul_inplace_transposed: k must be a multiple of %d", f16 ? 8 : 4);
+    CtxLock lock(dst->ctx);
+    hipStream_t st = dst->ctx->stream;
+    const int n = src->rows, k = src->cols, mrows = other->rows;
+    float *xf = nullptr, *yf = nullptr;
+    HIP_TRY(hipMalloc((void **)&xf, sizeof(float) * (size_t)n * k));
+    hipError_t e = hipMalloc((void **)&yf, sizeof(float) * (size_t)n * mrows);
+    if (e == hipSuccess) e = launch_convert(xf, 0, src->p, f16, (uint64_t)n * k, st);
+    for (int r = 0; e == hipSuccess && r < n; r++) {
+        GemvParams p{};
+        p.w = other->p;
+        p.w_is_f16 = f16;
+        p.x = xf + (size_t)r * k;
+        p.x_f16 = f16;
+        p.round_y = f16;
+        p.y = yf + (size_t)r * mrows;
+        p.n_rows = mrows;
+        p.k = k;
+        p.stream_weights = 0;
+        e = launch_gemv(p, kEpiStore, st);
+    }
+    if (e == hipSuccess) e = launch_convert(dst->p, f16, yf, 0, (uint64_t)n * mrows, st);
+    hipError_t e2 = hipStreamSynchronize(st);
+    if (xf) (void)hipFree(xf);
+    if (yf) (void)hipFree(yf);
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    return RLH_OK;
+}
+
+extern "C" int rlh_rmsnorm(rlh_tensor *y, const rlh_tensor *x, const rlh_tensor *w, double eps, int round_y) {
+    if (!y || !x || !w) return fail(RLH_ERR_INVALID, "rlh_rmsnorm: NULL argument");
+    if (x->dtype != RLH_F32 || y->dtype != RLH_F32 || w->dtype != RLH_F32) return fail(RLH_ERR_INVALID, "rlh_rmsnorm: f32 tensors only");
+    if (!same_shape(x, y) || w->rows != 1 || w->cols != x->cols) return fail(RLH_ERR_INVALID, "rlh_rmsnorm: shape mismatch");
+    CtxLock lock(y->ctx);
+    HIP_TRY(launch_rmsnorm_rows((float *)y->p, (const float *)x->p, (const float *)w->p, x->rows, x->cols, (float)eps, round_y, y->ctx->stream));
+    return RLH_OK;
+}
+
+extern "C" int rlh_rope_inplace(rlh_tensor *x, int n_heads, int head_dim, int pos) {
+    if (!x || x->dtype != RLH_F32 || n_heads <= 0 || head_dim <= 0 || (head_dim % 2) != 0 || pos < 0 || x->count() != (size_t)n_heads * head_dim) {
+        return fail(RLH_ERR_INVALID, "rlh_rope_inplace: bad argument");
+    }
+    CtxLock lock(x->ctx);
+    std::vector<float2> tab((size_t)head_dim / 2);
+    for (int j = 0; j < head_dim / 2; j++) {
+        const double freq = 1.0 / std::pow(10000.0, (double)j * 2.0 / (double)head_dim);
+        const double ang = freq * (double)pos;
+        tab[(size_t)j] = make_float2((float)std::cos(ang), (float)std::sin(ang));
+    }
+    float2 *dev = nullptr;
+    HIP_TRY(hipMalloc((void **)&dev, tab.size() * sizeof(float2)));
+    hipError_t e = hipMemcpyAsync(dev, tab.data(), tab.size() * sizeof(float2), hipMemcpyHostToDevice, x->ctx->stream);
+    if (e == hipSuccess) e = launch_rope_row((float *)x->p, n_heads, head_dim, dev, x->ctx->stream);
+    hipError_t e2 = hipStreamSynchronize(x->ctx->stream);
+    (void)hipFree(dev);
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    return RLH_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// synthetic inputs on the host
+// ------------------------------------------------------------------------------------------------
+extern "C" void rlh_synth_normal_f16(uint64_t seed, int kind, int layer, uint64_t first_index, uint64_t count, double std, uint16_t *out) {
+    const uint64_t key = synth_key(seed, SYNTH_STREAM_TENSOR(kind, layer));
+    unsigned nt = std::thread::hardware_concurrency();
+    if (nt > 16) nt = 16;
+    if (nt < 1 || count < (1u << 16)) nt = 1;
+    auto work = [=](uint64_t lo, uint64_t hi) {
+        uint64_t have = ~0ull; // pair whose deviates are in z0, z1
+        double z0 = 0.0, z1 = 0.0;
+        for (uint64_t i = lo; i < hi; i++) {
+            const uint64_t idx = first_index + i;
+            if ((idx >> 1) != have) {
+                have = idx >> 1;
+                synth_normal_pair(key, have, &z0, &z1);
+            }
+            out[i] = synth_scale_to_f16((idx & 1u) ? z1 : z0, std);
+        }
+    };
+    if (nt == 1) {
+        work(0, count);
+        return;
+    }
+    std::vector<std::thread> pool;
+    const uint64_t per = (count + nt - 1) / nt;
+    for (unsigned t = 0; t < nt; t++) {
+        const uint64_t lo = (uint64_t)t * per, hi = lo + per < count ? lo + per : count;
+        if (lo < hi) pool.emplace_back(work, lo, hi);
+    }
+    for (auto &th : pool) th.join();
+}
+
+extern "C" void rlh_synth_tokens(uint64_t seed, uint64_t first_index, uint64_t count, int32_t lo, int32_t hi, int32_t *out) {
+    const uint64_t key = synth_key(seed, SYNTH_STREAM_TOKENS);
+    for (uint64_t i = 0; i < count; i++) out[i] = synth_token(key, first_index + i, lo, hi);
+}

@@ -1,0 +1,99 @@
+// kernels.h -- host-side launch interface of the gfx950 kernels (internal to librllama_hip.so).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace rlh {
+
+enum GemvEpilogue {
+    kEpiStore = 0,   // y[c] = v
+    kEpiResAdd = 1,  // y[c] += v                      (wo and w2: the residual adds of transformer.rs:442, 445)
+    kEpiRopeKv = 2,  // fused wq|wk|wv: RoPE on q and k, q -> y, k/v -> KV cache at *pos
+    kEpiSilu = 3     // two matrices (w1, w3): y[c] = silu(v1) * v3   (transformer.rs:561-562)
+};
+
+// Device-resident scalars of the token loop.  Kernels read them from memory so that a recorded
+// sequence of launches can be replayed for the next token without new arguments.
+struct DecodeState {
+    int32_t pos;       // position of the token being processed (start_pos of transformer.rs:343)
+    int32_t token;     // its id
+    int32_t n_out;     // how many ids the argmax kernel has appended to out_tokens
+    int32_t pad;
+};
+
+struct GemvParams {
+    const void *w;            // [n_rows x k] row-major, f16 or f32
+    const void *w_b;          // kEpiSilu: second matrix (w3), same shape
+    const float *x;           // [k] f32
+    const float *norm_w;      // fused RMSNorm weight [k] or nullptr
+    float eps;
+    float *y;
+    int n_rows;
+    int k;
+    int w_is_f16;             // weight storage
+    int x_f16;                // 1: x (after the optional norm) is rounded to f16 before the product
+    int round_y;              // 1: product rounded to f16 precision (tensor.rs:1623-1643)
+    int stream_weights;       // 1: non-temporal weight loads
+    // kEpiRopeKv only
+    const DecodeState *state;
+    const float2 *freqs;      // [max_seq_len x head_dim/2] (cos, sin) as f32
+    void *cache_k;            // this layer's K cache [n_heads x max_seq_len x head_dim]
+    void *cache_v;
+    int cache_f16;
+    int dim;
+    int head_dim;
+    int max_seq_len;
+};
+
+hipError_t launch_gemv(const GemvParams &p, int epilogue, hipStream_t s);
+// bytes of dynamic LDS launch_gemv will request for a given k (for capability checks)
+size_t gemv_lds_bytes(int k, int w_is_f16, int x_f16);
+
+struct AttnDecodeParams {
+    const float *q;           // [n_heads x head_dim] f32 (after RoPE)
+    const void *cache_k;      // this layer: [n_heads x max_seq_len x head_dim]
+    const void *cache_v;
+    int cache_f16;
+    const DecodeState *state; // T = state->pos + 1
+    int n_heads;
+    int head_dim;
+    int max_seq_len;
+    int n_splits;             // grid.y; partial results are combined by the last block of each head
+    int chunk_cap;            // LDS score slots per block: >= ceil(T / n_splits) rounded up to 16
+    float *out;               // [n_heads x head_dim]
+    int round_out;            // f16 rounding point before wo (transformer.rs:793-796)
+    float *workspace;         // [n_heads x n_splits x (head_dim + 2)]
+    unsigned int *counters;   // [n_heads], zero between launches
+};
+
+hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s);
+
+hipError_t launch_embed(const void *table, int table_f16, int dim, const DecodeState *state, float *x, hipStream_t s);
+// argmax with TokenSampler's top_k = 1 behaviour (token_sampler.rs:112-147); writes state->token, appends to
+// out_tokens[state->n_out++] and advances state->pos.
+hipError_t launch_argmax_advance(const float *logits, int vocab, DecodeState *state, int32_t *out_tokens, int out_cap,
+                                 hipStream_t s);
+hipError_t launch_set_state(DecodeState *state, int pos, int token, int reset_out, hipStream_t s);
+hipError_t launch_reset_out(DecodeState *state, hipStream_t s);
+hipError_t launch_advance_pos(DecodeState *state, const int32_t *tokens_dev, int idx, hipStream_t s);
+
+// synthetic fills (synth.h)
+hipError_t launch_synth_fill(void *dst, int dst_f16, uint64_t n, uint64_t key, double std, hipStream_t s);
+hipError_t launch_fill_f32(float *dst, uint64_t n, float v, hipStream_t s);
+hipError_t launch_fill_u32(uint32_t *dst, uint64_t n, uint32_t v, hipStream_t s);
+
+// op level (OpenCLTensor's op set, tensor_opencl_support.rs:215-405)
+hipError_t launch_convert(void *dst, int dst_f16, const void *src, int src_f16, uint64_t n, hipStream_t s);
+hipError_t launch_transpose(void *dst, const void *src, int rows, int cols, int is_f16, hipStream_t s); // src [rows x cols]
+hipError_t launch_hadamard(void *dst, const void *src, uint64_t n, int is_f16, hipStream_t s);
+hipError_t launch_silu(void *dst, uint64_t n, int is_f16, hipStream_t s);
+hipError_t launch_rmsnorm_rows(float *y, const float *x, const float *w, int rows, int d, float eps, int round_y, hipStream_t s);
+hipError_t launch_rope_row(float *x, int n_heads, int head_dim, const float2 *freqs_at_pos, hipStream_t s);
+// KV-cache services (transformer.rs:180-197): shift positions left by `shifts` within each (head) plane
+hipError_t launch_cache_shift_left(void *cache, int is_f16, size_t planes, int max_seq_len, int head_dim, int shifts, hipStream_t s);
+// test hook: [head_dim x max_seq_len] f32 view of one head's plane
+hipError_t launch_cache_read(float *dst, const void *plane, int is_f16, int max_seq_len, int head_dim, hipStream_t s);
+
+} // namespace rlh
