@@ -70,6 +70,7 @@ class Context:
         return us.value
 
     def close(self) -> None:
+        """Ends the context.  Handles made from it are dead afterwards (their free() becomes a no-op)."""
         if getattr(self, "_h", None):
             self._lib.rlh_shutdown(self._h)
             self._h = None
@@ -132,7 +133,8 @@ class TransformerCaches:
 
     def free(self) -> None:
         if getattr(self, "_h", None):
-            self._lib.rlh_caches_free(self._h)
+            if self._model.ctx._h:
+                self._lib.rlh_caches_free(self._h)
             self._h = None
 
     def __del__(self):
@@ -241,7 +243,8 @@ class Transformer:
 
     def free(self) -> None:
         if getattr(self, "_h", None):
-            self._lib.rlh_model_free(self._h)
+            if self.ctx._h:
+                self._lib.rlh_model_free(self._h)
             self._h = None
 
     def __del__(self):
@@ -345,7 +348,8 @@ class Tensor:
 
     def free(self) -> None:
         if getattr(self, "_h", None):
-            self._lib.rlh_tensor_free(self._h)
+            if self.ctx._h:
+                self._lib.rlh_tensor_free(self._h)
             self._h = None
 
     def __del__(self):

@@ -98,7 +98,9 @@ struct rlh_model {
 };
 
 struct rlh_caches {
-    rlh_model *model = nullptr;
+    rlh_ctx *ctx = nullptr;
+    const rlh_model *model = nullptr; // identity only: never dereferenced (the model may be freed first)
+    int n_layers = 0, n_heads = 0, head_dim = 0, max_seq_len = 0;
     void *k = nullptr, *v = nullptr;
     size_t bytes_each = 0;
     int f16 = 0;
@@ -499,14 +501,19 @@ extern "C" int rlh_caches_create(rlh_model *m, rlh_caches **out) {
     *out = nullptr;
     CtxLock lock(m->ctx);
     rlh_caches *c = new rlh_caches();
+    c->ctx = m->ctx;
     c->model = m;
+    c->n_layers = m->prm.n_layers;
+    c->n_heads = m->prm.n_heads;
+    c->head_dim = m->head_dim;
+    c->max_seq_len = m->prm.max_seq_len;
     c->f16 = m->prm.force_f16 ? 1 : 0; // transformer.rs:138-142
-    c->bytes_each = (size_t)m->prm.n_layers * m->prm.n_heads * m->prm.max_seq_len * m->head_dim * (c->f16 ? 2 : 4);
+    c->bytes_each = (size_t)c->n_layers * c->n_heads * c->max_seq_len * c->head_dim * (c->f16 ? 2 : 4);
     hipError_t e = hipMalloc(&c->k, c->bytes_each);
     if (e == hipSuccess) e = hipMalloc(&c->v, c->bytes_each);
-    if (e == hipSuccess) e = hipMemsetAsync(c->k, 0, c->bytes_each, m->ctx->stream); // Tensor::zeros
-    if (e == hipSuccess) e = hipMemsetAsync(c->v, 0, c->bytes_each, m->ctx->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(m->ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(c->k, 0, c->bytes_each, c->ctx->stream); // Tensor::zeros
+    if (e == hipSuccess) e = hipMemsetAsync(c->v, 0, c->bytes_each, c->ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->ctx->stream);
     if (e != hipSuccess) {
         if (c->k) (void)hipFree(c->k);
         if (c->v) (void)hipFree(c->v);
@@ -520,7 +527,7 @@ extern "C" int rlh_caches_create(rlh_model *m, rlh_caches **out) {
 extern "C" int rlh_caches_true_clone(const rlh_caches *src, rlh_caches **out) {
     if (!src || !out) return fail(RLH_ERR_INVALID, "rlh_caches_true_clone: NULL argument");
     *out = nullptr;
-    rlh_ctx *ctx = src->model->ctx;
+    rlh_ctx *ctx = src->ctx;
     CtxLock lock(ctx);
     rlh_caches *c = new rlh_caches(*src);
     c->k = c->v = nullptr;
@@ -542,18 +549,17 @@ extern "C" int rlh_caches_true_clone(const rlh_caches *src, rlh_caches **out) {
 extern "C" int rlh_caches_shift_left(rlh_caches *c, int shifts) {
     if (!c || shifts < 0) return fail(RLH_ERR_INVALID, "rlh_caches_shift_left: bad argument");
     if (shifts == 0) return RLH_OK;
-    rlh_model *m = c->model;
-    CtxLock lock(m->ctx);
-    const size_t planes = (size_t)m->prm.n_layers * m->prm.n_heads;
-    HIP_TRY(launch_cache_shift_left(c->k, c->f16, planes, m->prm.max_seq_len, m->head_dim, shifts, m->ctx->stream));
-    HIP_TRY(launch_cache_shift_left(c->v, c->f16, planes, m->prm.max_seq_len, m->head_dim, shifts, m->ctx->stream));
+    CtxLock lock(c->ctx);
+    const size_t planes = (size_t)c->n_layers * c->n_heads;
+    HIP_TRY(launch_cache_shift_left(c->k, c->f16, planes, c->max_seq_len, c->head_dim, shifts, c->ctx->stream));
+    HIP_TRY(launch_cache_shift_left(c->v, c->f16, planes, c->max_seq_len, c->head_dim, shifts, c->ctx->stream));
     return RLH_OK;
 }
 
 extern "C" void rlh_caches_free(rlh_caches *c) {
     if (!c) return;
-    CtxLock lock(c->model->ctx);
-    (void)hipStreamSynchronize(c->model->ctx->stream);
+    CtxLock lock(c->ctx);
+    (void)hipStreamSynchronize(c->ctx->stream);
     if (c->k) (void)hipFree(c->k);
     if (c->v) (void)hipFree(c->v);
     delete c;
@@ -561,17 +567,17 @@ extern "C" void rlh_caches_free(rlh_caches *c) {
 
 extern "C" int rlh_caches_read(const rlh_caches *c, int layer, int head, int which, float *host_out) {
     if (!c || !host_out) return fail(RLH_ERR_INVALID, "rlh_caches_read: NULL argument");
-    rlh_model *m = c->model;
-    if (layer < 0 || layer >= m->prm.n_layers || head < 0 || head >= m->prm.n_heads) return fail(RLH_ERR_INVALID, "rlh_caches_read: index out of range");
-    CtxLock lock(m->ctx);
-    const size_t per_plane = (size_t)m->prm.max_seq_len * m->head_dim;
-    const size_t off = ((size_t)layer * m->prm.n_heads + head) * per_plane * (c->f16 ? 2 : 4);
+    if (layer < 0 || layer >= c->n_layers || head < 0 || head >= c->n_heads) return fail(RLH_ERR_INVALID, "rlh_caches_read: index out of range");
+    CtxLock lock(c->ctx);
+    hipStream_t st = c->ctx->stream;
+    const size_t per_plane = (size_t)c->max_seq_len * c->head_dim;
+    const size_t off = ((size_t)layer * c->n_heads + head) * per_plane * (c->f16 ? 2 : 4);
     const char *plane = (const char *)(which ? c->v : c->k) + off;
     float *tmp = nullptr;
     HIP_TRY(hipMalloc((void **)&tmp, per_plane * 4));
-    hipError_t e = launch_cache_read(tmp, plane, c->f16, m->prm.max_seq_len, m->head_dim, m->ctx->stream);
-    if (e == hipSuccess) e = hipMemcpyAsync(host_out, tmp, per_plane * 4, hipMemcpyDeviceToHost, m->ctx->stream);
-    hipError_t e2 = hipStreamSynchronize(m->ctx->stream);
+    hipError_t e = launch_cache_read(tmp, plane, c->f16, c->max_seq_len, c->head_dim, st);
+    if (e == hipSuccess) e = hipMemcpyAsync(host_out, tmp, per_plane * 4, hipMemcpyDeviceToHost, st);
+    hipError_t e2 = hipStreamSynchronize(st);
     (void)hipFree(tmp);
     HIP_TRY(e);
     HIP_TRY(e2);
