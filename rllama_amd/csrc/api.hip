@@ -82,14 +82,15 @@ struct rlh_model {
     std::vector<Layer> layers;
     float2 *freqs = nullptr;
     // activations of one token step
-    float *x = nullptr, *q = nullptr, *att = nullptr, *mh = nullptr, *logits = nullptr;
+    // x: residual stream entering a layer; h: after the attention block; att: attention output; att_o / ffn_o:
+    // outputs of wo / w2 (added to the stream in the next kernel's prologue)
+    float *x = nullptr, *h = nullptr, *q = nullptr, *att = nullptr, *att_o = nullptr, *mh = nullptr, *ffn_o = nullptr, *logits = nullptr;
     DecodeState *state = nullptr;
     int32_t *out_tokens = nullptr;
     int out_cap = 0;
     int32_t *prompt_dev = nullptr;
     int prompt_cap = 0;
     float *attn_ws = nullptr;
-    unsigned int *attn_counters = nullptr;
     int max_splits = 16;
     int stream_weights = 1;
     // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
@@ -286,7 +287,10 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     m->out_cap = prm->max_seq_len + 1;
     m->prompt_cap = prm->max_seq_len;
     B((void **)&m->x, sizeof(float) * d);
+    B((void **)&m->h, sizeof(float) * d);
     B((void **)&m->q, sizeof(float) * d);
+    B((void **)&m->att_o, sizeof(float) * d);
+    B((void **)&m->ffn_o, sizeof(float) * d);
     B((void **)&m->att, sizeof(float) * d);
     B((void **)&m->mh, sizeof(float) * F);
     B((void **)&m->logits, sizeof(float) * V);
@@ -294,7 +298,6 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     B((void **)&m->out_tokens, sizeof(int32_t) * m->out_cap);
     B((void **)&m->prompt_dev, sizeof(int32_t) * m->prompt_cap);
     B((void **)&m->attn_ws, sizeof(float) * (size_t)prm->n_heads * m->max_splits * (hd + 2));
-    B((void **)&m->attn_counters, sizeof(unsigned int) * prm->n_heads);
     if (rc == RLH_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(RLH_ERR_HIP, "rlh_model_create: hipDeviceSynchronize failed");
     if (rc != RLH_OK) {
         rlh_model_free(m);
@@ -320,7 +323,7 @@ extern "C" void rlh_model_free(rlh_model *m) {
     free_weight(m->tok_emb);
     free_weight(m->norm);
     free_weight(m->output);
-    void *bufs[] = {m->freqs, m->x, m->q, m->att, m->mh, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws, m->attn_counters};
+    void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -587,15 +590,13 @@ extern "C" int rlh_caches_read(const rlh_caches *c, int layer, int head, int whi
 // ------------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------------
-static void attn_config(const rlh_model *m, int T, int *splits, int *chunk_cap) {
-    // One block per (head, split).  Aim for chunks of >= 64 positions and at most max_splits splits.
-    int S = (T + 63) / 64;
+static int attn_splits(const rlh_model *m, int T) {
+    // One block per (head, split).  A block streams its share of the cache alone, so short sequences stay
+    // in one block per head; longer ones are cut into chunks of about 256 positions.
+    int S = (T + 255) / 256;
     if (S < 1) S = 1;
     if (S > m->max_splits) S = m->max_splits;
-    int chunk = (T + S - 1) / S;
-    chunk = (chunk + 15) & ~15;
-    *splits = S;
-    *chunk_cap = chunk;
+    return S;
 }
 
 enum StepKernel { kStepQkv = 0, kStepAttn = 1, kStepWo = 2, kStepW13 = 3, kStepW2 = 4, kStepHead = 5 };
@@ -614,13 +615,16 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
     g.x_f16 = f16;
     g.round_y = f16;
     g.eps = eps;
+    // The stream enters layer l in m->x (l == 0: the embedding row) or as m->h + m->ffn_o of layer l - 1.
     if (which == kStepHead) {
-        // final norm + output head: f32 activations, no rounding (transformer.rs:378-381; tensor.rs:1837-1918)
+        // last residual add + final norm + output head: f32 activations, no rounding
+        // (transformer.rs:445, 378-381; tensor.rs:1837-1918)
         GemvParams p{};
         p.stream_weights = m->stream_weights;
         p.w = m->output.p;
         p.w_is_f16 = m->output.f16;
-        p.x = m->x;
+        p.x = m->h;
+        p.x_add = m->ffn_o;
         p.x_f16 = 0;
         p.round_y = 0;
         p.norm_w = (const float *)m->norm.p;
@@ -638,10 +642,17 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
     void *cv = (char *)c->v + (size_t)l * layer_elems * ces;
     switch (which) {
     case kStepQkv: {
-        // attention_norm + wq|wk|wv + RoPE + cache write (transformer.rs:432, 665-668, 694-725, 751-761)
+        // (previous layer's second residual add, transformer.rs:445) + attention_norm + wq|wk|wv + RoPE + cache
+        // write (transformer.rs:432, 665-668, 694-725, 751-761)
         GemvParams p = g;
         p.w = L.wqkv.p;
-        p.x = m->x;
+        if (l == 0) {
+            p.x = m->x;
+        } else {
+            p.x = m->h;
+            p.x_add = m->ffn_o;
+            p.x_out = m->x;
+        }
         p.norm_w = (const float *)L.attn_norm.p;
         p.y = m->q;
         p.n_rows = 3 * d;
@@ -659,8 +670,6 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
     }
     case kStepAttn: {
         // scores, softmax, P.V (transformer.rs:762-779) + f16 rounding point before wo (:793-796)
-        int splits, chunk_cap;
-        attn_config(m, T_host, &splits, &chunk_cap);
         AttnDecodeParams a{};
         a.q = m->q;
         a.cache_k = ck;
@@ -670,32 +679,32 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         a.n_heads = P.n_heads;
         a.head_dim = m->head_dim;
         a.max_seq_len = P.max_seq_len;
-        a.n_splits = splits;
-        a.chunk_cap = chunk_cap;
+        a.n_splits = attn_splits(m, T_host);
         a.out = m->att;
         a.round_out = f16;
         a.workspace = m->attn_ws;
-        a.counters = m->attn_counters;
         HIP_TRY(launch_attn_decode(a, st));
         break;
     }
     case kStepWo: {
-        // wo + residual (transformer.rs:783-819, 442)
+        // wo (transformer.rs:783-819); its output joins the stream in the next kernel
         GemvParams p = g;
         p.w = L.wo.p;
         p.x = m->att;
-        p.y = m->x;
+        p.y = m->att_o;
         p.n_rows = d;
         p.k = d;
-        HIP_TRY(launch_gemv(p, kEpiResAdd, st));
+        HIP_TRY(launch_gemv(p, kEpiStore, st));
         break;
     }
     case kStepW13: {
-        // ffn_norm + w1|w3 + SiLU * gate (transformer.rs:443, 537-565)
+        // h = x + att_out (transformer.rs:442) + ffn_norm + w1|w3 + SiLU * gate (transformer.rs:443, 537-565)
         GemvParams p = g;
         p.w = L.w1.p;
         p.w_b = L.w3.p;
         p.x = m->x;
+        p.x_add = m->att_o;
+        p.x_out = m->h;
         p.norm_w = (const float *)L.ffn_norm.p;
         p.y = m->mh;
         p.n_rows = F;
@@ -704,14 +713,14 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         break;
     }
     case kStepW2: {
-        // w2 + residual (transformer.rs:568-570, 445)
+        // w2 (transformer.rs:568-570); its output joins the stream in the next kernel
         GemvParams p = g;
         p.w = L.w2.p;
         p.x = m->mh;
-        p.y = m->x;
+        p.y = m->ffn_o;
         p.n_rows = d;
         p.k = F;
-        HIP_TRY(launch_gemv(p, kEpiResAdd, st));
+        HIP_TRY(launch_gemv(p, kEpiStore, st));
         break;
     }
     default: return fail(RLH_ERR_INVALID, "unknown step kernel %d", which);

@@ -96,4 +96,15 @@ __device__ __forceinline__ uint4_t load16(const void *p) {
     }
 }
 
+// One interleaved RoPE pair (transformer.rs:844-847): four products and two sums, each rounded to f32 (no FMA).
+__device__ __forceinline__ void rope_pair(float re, float im, float2 f, float &ore, float &oim) {
+#pragma clang fp contract(off)
+    float p0 = re * f.x;
+    float p1 = im * f.y;
+    float p2 = re * f.y;
+    float p3 = im * f.x;
+    ore = p0 - p1;
+    oim = p2 + p3;
+}
+
 } // namespace rlh

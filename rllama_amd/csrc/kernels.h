@@ -9,7 +9,6 @@ namespace rlh {
 
 enum GemvEpilogue {
     kEpiStore = 0,   // y[c] = v
-    kEpiResAdd = 1,  // y[c] += v                      (wo and w2: the residual adds of transformer.rs:442, 445)
     kEpiRopeKv = 2,  // fused wq|wk|wv: RoPE on q and k, q -> y, k/v -> KV cache at *pos
     kEpiSilu = 3     // two matrices (w1, w3): y[c] = silu(v1) * v3   (transformer.rs:561-562)
 };
@@ -27,6 +26,9 @@ struct GemvParams {
     const void *w;            // [n_rows x k] row-major, f16 or f32
     const void *w_b;          // kEpiSilu: second matrix (w3), same shape
     const float *x;           // [k] f32
+    const float *x_add;       // optional [k]: the product's input is x + x_add (the residual adds of
+                              // transformer.rs:442, 445 happen in the consumer's prologue)
+    float *x_out;             // optional [k]: block 0 stores x + x_add here (must not alias x or x_add)
     const float *norm_w;      // fused RMSNorm weight [k] or nullptr
     float eps;
     float *y;
@@ -36,6 +38,7 @@ struct GemvParams {
     int x_f16;                // 1: x (after the optional norm) is rounded to f16 before the product
     int round_y;              // 1: product rounded to f16 precision (tensor.rs:1623-1643)
     int stream_weights;       // 1: non-temporal weight loads
+    int rows_per_wave;        // set by launch_gemv
     // kEpiRopeKv only
     const DecodeState *state;
     const float2 *freqs;      // [max_seq_len x head_dim/2] (cos, sin) as f32
@@ -60,12 +63,10 @@ struct AttnDecodeParams {
     int n_heads;
     int head_dim;
     int max_seq_len;
-    int n_splits;             // grid.y; partial results are combined by the last block of each head
-    int chunk_cap;            // LDS score slots per block: >= ceil(T / n_splits) rounded up to 16
+    int n_splits;             // grid.y; with more than one, a second small kernel merges the partial results
     float *out;               // [n_heads x head_dim]
     int round_out;            // f16 rounding point before wo (transformer.rs:793-796)
-    float *workspace;         // [n_heads x n_splits x (head_dim + 2)]
-    unsigned int *counters;   // [n_heads], zero between launches
+    float *workspace;         // [n_heads x n_splits x (head_dim + 2)], needed when n_splits > 1
 };
 
 hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s);
