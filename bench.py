@@ -90,6 +90,12 @@ def main() -> int:
     ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-iters", type=int, default=320)
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="skip the token loop and the CPU baseline: only the per-kernel timing loops (short runs for "
+                         "rocprofv3 --pmc passes)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain copy kernel over 1 GiB of f32 (reads 1 GiB, writes 1 GiB per launch): "
+                         "the known-size reference for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (batch-1 decode of one model resident in one device's HBM); "
@@ -97,6 +103,18 @@ def main() -> int:
         return 2
 
     import rllama_amd as ra
+
+    if args.calibrate_copy:
+        ctx = ra.Context(0)
+        rows, cols = 16384, 16384  # 2^28 f32 = 1 GiB
+        src = ra.Tensor.zeros(ctx, rows, cols, ra.TensorDType.Float32)
+        for _ in range(4):
+            dst = src.clone()     # one convert_kernel<float, float> launch: 1 GiB read + 1 GiB written
+            dst.free()
+        ctx.sync()
+        print(json.dumps({"calibration": "convert_kernel<float,float> copy", "launches": 4, "bytes_read_per_launch": rows * cols * 4,
+                          "bytes_written_per_launch": rows * cols * 4}))
+        return 0
 
     dim, n_layers, n_heads, ffn, vocab, n_prompt, dflt_steps = CONFIGS[args.config]
     K = args.steps if args.steps is not None else dflt_steps
@@ -109,6 +127,16 @@ def main() -> int:
     model = ra.Transformer(ctx, dim, n_layers, n_heads, ffn, vocab, max_seq, 1e-6, ds)
     model.fill_synthetic(seed=0, std=0.02)
     prompt = ra.synth_tokens(0, n_prompt, 3, vocab)
+
+    if args.kernels_only:
+        caches = model.make_caches()
+        T_mid = n_prompt + K // 2
+        out = {"kernels_only": True, "T": T_mid, "kernels": {}}
+        for which, name in enumerate(ra.Transformer.STEP_KERNELS):
+            us, nbytes = model.time_kernel(which, T_mid, args.kernel_iters, caches)
+            out["kernels"][name] = {"us": round(us, 2), "bytes": nbytes}
+        print(json.dumps(out))
+        return 0
 
     # ---- warmup: W untimed decode steps (own caches, same prompt) ----
     cw = model.make_caches()

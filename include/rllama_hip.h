@@ -109,6 +109,11 @@ int  rlh_model_get_tensor(rlh_model *model, int kind, int layer, void *host_out,
  * embedding and head i.i.d. N(0, std^2) rounded to f16, norm weights 1.0.  Bit-identical to
  * rlh_synth_normal_f16 on the host.  (No reference counterpart: the reference only loads files.) */
 int  rlh_model_fill_synthetic(rlh_model *model, uint64_t seed, double std);
+/* How a multi-token forward (n > 1 at start_pos == 0, src/transformer.rs:343-383) is executed.  0 (default): every
+ * projection as one matrix-core GEMM over all n rows and attention as batched GEMMs around a causal softmax
+ * (f16 mode; f32 mode has no f16 operands for the matrix cores and always uses mode 1).  1: token by token with
+ * the decode kernels.  Both give the reference's result up to the order of fp32 additions. */
+int  rlh_model_set_prefill_mode(rlh_model *model, int mode);
 /* The layer split rule of src/transformer.rs:262-279: last_layer_on_gpu = round(p * (n_layers - 1)).
  * Reports it; all layers run on the device regardless (nothing is left on the host). */
 int  rlh_model_layers_on_gpu(const rlh_model *model, int *last_layer_on_gpu);

@@ -186,6 +186,10 @@ class Transformer:
     def fill_synthetic(self, seed: int = 0, std: float = 0.02) -> None:
         check(self._lib.rlh_model_fill_synthetic(self._h, seed, std))
 
+    def set_prefill_mode(self, token_by_token: bool) -> None:
+        """False (default): matrix-core prefill for n > 1 in f16 mode.  True: the decode kernels for every prompt token."""
+        check(self._lib.rlh_model_set_prefill_mode(self._h, 1 if token_by_token else 0))
+
     def last_layer_on_gpu(self) -> int:
         v = C.c_int()
         check(self._lib.rlh_model_layers_on_gpu(self._h, C.byref(v)))

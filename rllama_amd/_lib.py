@@ -5,7 +5,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "librllama_hip.so")
+# RLLAMA_HIP_LIB names another build of the same library (e.g. a variant under test)
+LIB_PATH = os.environ.get("RLLAMA_HIP_LIB") or os.path.join(HERE, "librllama_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(HERE), "include", "rllama_hip.h")
 
 
@@ -47,6 +48,7 @@ SIGNATURES = {
     "rlh_model_set_tensor": (C.c_int, [_vp, C.c_int, C.c_int, _vp, C.c_int, C.c_int, C.c_int]),
     "rlh_model_get_tensor": (C.c_int, [_vp, C.c_int, C.c_int, _vp, C.c_int, C.c_int, C.c_int]),
     "rlh_model_fill_synthetic": (C.c_int, [_vp, C.c_uint64, C.c_double]),
+    "rlh_model_set_prefill_mode": (C.c_int, [_vp, C.c_int]),
     "rlh_model_layers_on_gpu": (C.c_int, [_vp, _ip]),
     "rlh_model_decode_bytes": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_uint64)]),
     "rlh_caches_create": (C.c_int, [_vp, _vpp]),

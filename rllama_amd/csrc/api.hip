@@ -73,6 +73,21 @@ struct Layer {
     Weight wo, w1, w2, w3, attn_norm, ffn_norm;
 };
 
+// Work buffers of a multi-token forward (prefill); grown on demand, kept for the next call.
+struct PrefillScratch {
+    int n_cap = 0;       // rows the buffers are sized for
+    int t_pad = 0;       // n_cap rounded up to 8: row stride of scores / probabilities / transposed V
+    float *x = nullptr, *h = nullptr, *scores = nullptr, *o = nullptr;
+    void *xn = nullptr, *qkv = nullptr, *q_hi = nullptr, *q_lo = nullptr, *v_t = nullptr, *p_hi = nullptr, *p_lo = nullptr, *a = nullptr;
+    void *g = nullptr, *u = nullptr, *mm = nullptr;
+    void release() {
+        void *all[] = {x, h, scores, o, xn, qkv, q_hi, q_lo, v_t, p_hi, p_lo, a, g, u, mm};
+        for (void *b : all)
+            if (b) (void)hipFree(b);
+        *this = PrefillScratch();
+    }
+};
+
 struct rlh_model {
     rlh_ctx *ctx = nullptr;
     rlh_model_params prm;
@@ -93,6 +108,8 @@ struct rlh_model {
     float *attn_ws = nullptr;
     int max_splits = 16;
     int stream_weights = 1;
+    PrefillScratch pf;
+    int prefill_mode = 0; // 0: matrix-core prefill where available (f16 mode), 1: token by token
     // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
     int next_pos = -1;
     rlh_caches *greedy_caches = nullptr;
@@ -323,6 +340,7 @@ extern "C" void rlh_model_free(rlh_model *m) {
     free_weight(m->tok_emb);
     free_weight(m->norm);
     free_weight(m->output);
+    m->pf.release();
     void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
@@ -465,6 +483,12 @@ extern "C" int rlh_model_fill_synthetic(rlh_model *m, uint64_t seed, double std)
         L.wo.loaded = L.w1.loaded = L.w2.loaded = L.w3.loaded = L.attn_norm.loaded = L.ffn_norm.loaded = true;
     }
     HIP_TRY(hipStreamSynchronize(st));
+    return RLH_OK;
+}
+
+extern "C" int rlh_model_set_prefill_mode(rlh_model *m, int mode) {
+    if (!m || (mode != 0 && mode != 1)) return fail(RLH_ERR_INVALID, "rlh_model_set_prefill_mode: bad argument");
+    m->prefill_mode = mode;
     return RLH_OK;
 }
 
@@ -742,6 +766,158 @@ static int enqueue_token_step(rlh_model *m, rlh_caches *c, int T_host, bool with
     return RLH_OK;
 }
 
+static int ensure_prefill_scratch(rlh_model *m, int n) {
+    PrefillScratch &S = m->pf;
+    if (n <= S.n_cap) return RLH_OK;
+    S.release();
+    const size_t d = (size_t)m->prm.dim, F = (size_t)m->prm.ffn_hidden, H = (size_t)m->prm.n_heads, hd = (size_t)m->head_dim;
+    const size_t N = (size_t)n, tp = (N + 7) & ~(size_t)7;
+    hipError_t e = hipSuccess;
+    auto A = [&](void **p, size_t bytes) {
+        if (e != hipSuccess) return;
+        e = hipMalloc(p, bytes);
+        if (e == hipSuccess) e = hipMemsetAsync(*p, 0, bytes, m->ctx->stream); // padding must hold finite values
+    };
+    A((void **)&S.x, N * d * 4);
+    A((void **)&S.h, N * d * 4);
+    A((void **)&S.xn, N * d * 2);
+    A((void **)&S.qkv, N * 3 * d * 2);
+    A((void **)&S.q_hi, N * d * 2);
+    A((void **)&S.q_lo, N * d * 2);
+    A((void **)&S.v_t, H * hd * tp * 2);
+    A((void **)&S.scores, H * N * tp * 4);
+    A((void **)&S.p_hi, H * N * tp * 2);
+    A((void **)&S.p_lo, H * N * tp * 2);
+    A((void **)&S.o, N * d * 4);
+    A((void **)&S.a, N * d * 2);
+    A((void **)&S.g, N * F * 2);
+    A((void **)&S.u, N * F * 2);
+    A((void **)&S.mm, N * F * 2);
+    if (e == hipSuccess) e = hipStreamSynchronize(m->ctx->stream);
+    if (e != hipSuccess) {
+        S.release();
+        return fail(e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "prefill work buffers for %d tokens: %s", n, hipGetErrorString(e));
+    }
+    S.n_cap = n;
+    S.t_pad = (int)tp;
+    return RLH_OK;
+}
+
+// Multi-token forward at start_pos == 0 in f16 mode: every projection is one matrix-core GEMM over all n rows
+// (transformer.rs:694-702, 783-815, 551-570 with seq_len > 1), attention is two batched GEMMs per head around a
+// causal softmax (transformer.rs:762-779).  Leaves the last row's logits in m->logits and the KV cache filled.
+static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n) {
+    int rc = ensure_prefill_scratch(m, n);
+    if (rc != RLH_OK) return rc;
+    hipStream_t st = m->ctx->stream;
+    const rlh_model_params &P = m->prm;
+    PrefillScratch &S = m->pf;
+    const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size, H = P.n_heads, hd = m->head_dim;
+    const int tp = (n + 7) & ~7; // row stride of this call's scores / probabilities / transposed V
+    const float eps = (float)P.norm_eps;
+    HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
+    HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));
+    HIP_TRY(launch_embed_rows(m->tok_emb.p, m->tok_emb.f16, m->prompt_dev, n, d, S.x, st));
+    const size_t layer_elems = (size_t)H * P.max_seq_len * hd;
+    auto gemm = [&](const void *a, int lda, const void *b, int ldb, void *cc, int ldc, int mm, int nn, int kk, int epi, const float *res) -> int {
+        GemmParams g{};
+        g.a = (const _Float16 *)a;
+        g.b = (const _Float16 *)b;
+        g.c = cc;
+        g.residual = res;
+        g.m = mm;
+        g.n = nn;
+        g.k = kk;
+        g.lda = lda;
+        g.ldb = ldb;
+        g.ldc = ldc;
+        g.batch = 1;
+        HIP_TRY(launch_gemm_f16(g, epi, st));
+        return RLH_OK;
+    };
+    for (int l = 0; l < P.n_layers; l++) {
+        Layer &L = m->layers[(size_t)l];
+        char *ck = (char *)c->k + (size_t)l * layer_elems * 2;
+        char *cv = (char *)c->v + (size_t)l * layer_elems * 2;
+        HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.x, (const float *)L.attn_norm.p, n, d, eps, st));
+        if ((rc = gemm(S.xn, d, L.wqkv.p, d, S.qkv, 3 * d, n, 3 * d, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
+        PrefillRopeParams rp{};
+        rp.qkv = S.qkv;
+        rp.freqs = m->freqs;
+        rp.q_hi = S.q_hi;
+        rp.q_lo = S.q_lo;
+        rp.cache_k = ck;
+        rp.cache_v = cv;
+        rp.cache_f16 = 1;
+        rp.v_t = S.v_t;
+        rp.n = n;
+        rp.dim = d;
+        rp.head_dim = hd;
+        rp.max_seq_len = P.max_seq_len;
+        rp.t_pad = tp;
+        HIP_TRY(launch_rope_kv_prefill(rp, st));
+        // scores[h] = q[h] . K[h]^T, accumulated over the hi and lo parts of q
+        for (int part = 0; part < 2; part++) {
+            GemmParams g{};
+            g.a = (const _Float16 *)(part == 0 ? S.q_hi : S.q_lo);
+            g.b = (const _Float16 *)ck;
+            g.c = S.scores;
+            g.m = n;
+            g.n = n;
+            g.k = hd;
+            g.lda = hd;
+            g.ldb = hd;
+            g.ldc = tp;
+            g.batch = H;
+            g.stride_a = (size_t)n * hd;
+            g.stride_b = (size_t)P.max_seq_len * hd;
+            g.stride_c = (size_t)n * tp;
+            g.accumulate = part;
+            HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
+        }
+        HIP_TRY(launch_causal_softmax(S.scores, S.p_hi, S.p_lo, H, n, tp, hd, st));
+        // out[h] = P[h] . V[h], accumulated over the hi and lo parts of P
+        for (int part = 0; part < 2; part++) {
+            GemmParams g{};
+            g.a = (const _Float16 *)(part == 0 ? S.p_hi : S.p_lo);
+            g.b = (const _Float16 *)S.v_t;
+            g.c = S.o;
+            g.m = n;
+            g.n = hd;
+            g.k = tp;
+            g.lda = tp;
+            g.ldb = tp;
+            g.ldc = hd;
+            g.batch = H;
+            g.stride_a = (size_t)n * tp;
+            g.stride_b = (size_t)hd * tp;
+            g.stride_c = (size_t)n * hd;
+            g.accumulate = part;
+            HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
+        }
+        HIP_TRY(launch_attn_out_f16(S.o, S.a, n, H, hd, st));
+        if ((rc = gemm(S.a, d, L.wo.p, d, S.h, d, n, d, d, kGemmEpiResAddF32, S.x)) != RLH_OK) return rc;     // h = x + wo(att)
+        HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.h, (const float *)L.ffn_norm.p, n, d, eps, st));
+        if ((rc = gemm(S.xn, d, L.w1.p, d, S.g, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
+        if ((rc = gemm(S.xn, d, L.w3.p, d, S.u, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
+        HIP_TRY(launch_silu_mul_f16(S.g, S.u, S.mm, (size_t)n * F, st));
+        if ((rc = gemm(S.mm, F, L.w2.p, F, S.x, d, n, d, F, kGemmEpiResAddF32, S.h)) != RLH_OK) return rc;    // x = h + w2(...)
+    }
+    // final norm + output head on the last row only (transformer.rs:378-381)
+    GemvParams p{};
+    p.stream_weights = m->stream_weights;
+    p.w = m->output.p;
+    p.w_is_f16 = m->output.f16;
+    p.x = S.x + (size_t)(n - 1) * d;
+    p.norm_w = (const float *)m->norm.p;
+    p.eps = eps;
+    p.y = m->logits;
+    p.n_rows = V;
+    p.k = d;
+    HIP_TRY(launch_gemv(p, kEpiStore, st));
+    return RLH_OK;
+}
+
 static int check_forward_args(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, const char *who) {
     if (!m || !c || !tokens) return fail(RLH_ERR_INVALID, "%s: NULL argument", who);
     if (c->model != m) return fail(RLH_ERR_STATE, "%s: caches belong to another model", who);
@@ -764,6 +940,7 @@ static int enqueue_forward(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     hipStream_t st = m->ctx->stream;
     m->next_pos = -1;
     m->greedy_caches = nullptr;
+    if (n > 1 && m->prm.force_f16 && m->prefill_mode == 0) return enqueue_prefill(m, c, tokens, n);
     HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
     HIP_TRY(launch_set_state(m->state, start_pos, tokens[0], 1, st));
     for (int i = 0; i < n; i++) {
@@ -1102,7 +1279,8 @@ static int same_shape(const rlh_tensor *a, const rlh_tensor *b) { return a->rows
 extern "C" int rlh_copy_inplace(rlh_tensor *dst, const rlh_tensor *src) {
     if (!dst || !src || !same_shape(dst, src)) return fail(RLH_ERR_INVALID, "rlh_copy_inplace: shape/dtype mismatch");
     CtxLock lock(dst->ctx);
-    HIP_TRY(hipMemcpyAsync(dst->p, src->p, dst->count() * dst->esize(), hipMemcpyDeviceToDevice, dst->ctx->stream));
+    // a plain copy kernel (the reference's copy_inplace is a kernel too); also the calibration point for HBM counters
+    HIP_TRY(launch_convert(dst->p, dst->dtype == RLH_F16, src->p, src->dtype == RLH_F16, dst->count(), dst->ctx->stream));
     return RLH_OK;
 }
 
@@ -1161,6 +1339,22 @@ extern "C" int rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tens
     CtxLock lock(dst->ctx);
     hipStream_t st = dst->ctx->stream;
     const int n = src->rows, k = src->cols, mrows = other->rows;
+    if (f16 && n > 1) {
+        // more than one row of f16: the matrix-core GEMM (f32 operands keep the per-row path below)
+        GemmParams g{};
+        g.a = (const _Float16 *)src->p;
+        g.b = (const _Float16 *)other->p;
+        g.c = dst->p;
+        g.m = n;
+        g.n = mrows;
+        g.k = k;
+        g.lda = k;
+        g.ldb = k;
+        g.ldc = mrows;
+        g.batch = 1;
+        HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
+        return RLH_OK;
+    }
     float *xf = nullptr, *yf = nullptr;
     HIP_TRY(hipMalloc((void **)&xf, sizeof(float) * (size_t)n * k));
     hipError_t e = hipMalloc((void **)&yf, sizeof(float) * (size_t)n * mrows);

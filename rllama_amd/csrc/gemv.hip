@@ -23,9 +23,19 @@
 
 namespace rlh {
 
-constexpr int kGemvWaves = 4;
+// Launch shape (overridable at compile time for tuning runs).
+#ifndef RLH_GEMV_WAVES
+#define RLH_GEMV_WAVES 4
+#endif
+#ifndef RLH_GEMV_TARGET_WAVES
+#define RLH_GEMV_TARGET_WAVES 2048 // 256 CUs x 8 resident wavefronts
+#endif
+#ifndef RLH_GEMV_BURST
+#define RLH_GEMV_BURST 8
+#endif
+constexpr int kGemvWaves = RLH_GEMV_WAVES;
 constexpr int kGemvThreads = kGemvWaves * kWave;
-constexpr int kGemvTargetWaves = 2048; // 256 CUs x 8 resident wavefronts
+constexpr int kGemvTargetWaves = RLH_GEMV_TARGET_WAVES;
 
 template <typename WT>
 struct WVec;
@@ -90,7 +100,7 @@ __device__ __forceinline__ float wave_sum_lane63(float v) {
     return v;
 }
 
-constexpr int kGemvBurst = 8;       // 16-byte loads per lane issued back to back before they are consumed
+constexpr int kGemvBurst = RLH_GEMV_BURST; // 16-byte loads per lane issued back to back before they are consumed
 constexpr int kGemvPrologueVecs = 8; // float4 loads per thread per prologue batch (one batch covers k <= 8192)
 
 template <typename WT, typename XT, int kEpi, bool kStream>

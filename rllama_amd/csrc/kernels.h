@@ -71,6 +71,44 @@ struct AttnDecodeParams {
 
 hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s);
 
+// ---- prefill: C = A * B^T on the matrix cores (gemm.hip) ----
+enum GemmEpilogue {
+    kGemmEpiF16 = 0,        // C f16 = round(acc)                      (projection outputs, tensor.rs:1623-1643)
+    kGemmEpiF32 = 1,        // C f32 = acc, or += acc when accumulate  (attention scores / P.V partial products)
+    kGemmEpiResAddF32 = 2   // C f32 = residual + f16r(acc)            (wo and w2 followed by transformer.rs:442 / :445)
+};
+
+struct GemmParams {
+    const _Float16 *a;      // [m x k], row stride lda
+    const _Float16 *b;      // [n x k], row stride ldb
+    void *c;                // [m x n], row stride ldc
+    const float *residual;  // kGemmEpiResAddF32: [m x n], row stride ldc
+    int m, n, k;
+    int lda, ldb, ldc;
+    int batch;              // grid.z; element strides between batch items:
+    size_t stride_a, stride_b, stride_c;
+    int accumulate;         // kGemmEpiF32 only
+};
+
+hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s);
+
+// ---- prefill: element-wise kernels around the GEMMs (prefill.hip) ----
+struct PrefillRopeParams {
+    const void *qkv;        // [n x 3 dim] f16
+    const float2 *freqs;    // [max_seq_len x head_dim/2]
+    void *q_hi, *q_lo;      // [n_heads][n][head_dim] f16
+    void *cache_k, *cache_v; // this layer: [n_heads][max_seq_len][head_dim]
+    int cache_f16;
+    void *v_t;              // [n_heads][head_dim][t_pad] f16
+    int n, dim, head_dim, max_seq_len, t_pad;
+};
+hipError_t launch_embed_rows(const void *table, int table_f16, const int32_t *tokens_dev, int n, int dim, float *x, hipStream_t s);
+hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s);
+hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s);
+hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int head_dim, hipStream_t s);
+hipError_t launch_attn_out_f16(const float *o, void *a, int n, int n_heads, int head_dim, hipStream_t s);
+hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s);
+
 hipError_t launch_embed(const void *table, int table_f16, int dim, const DecodeState *state, float *x, hipStream_t s);
 // argmax with TokenSampler's top_k = 1 behaviour (token_sampler.rs:112-147); writes state->token, appends to
 // out_tokens[state->n_out++] and advances state->pos.

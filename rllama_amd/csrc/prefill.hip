@@ -1,0 +1,175 @@
+// prefill.hip -- the element-wise kernels around the matrix-core GEMMs of a multi-token forward at
+// start_pos == 0 (the only multi-token call the reference supports: its mask is n x n, transformer.rs:350-357).
+//
+// Rounding points are the reference's (Noeda/rllama): RMSNorm output -> f16 (transformer.rs:665-668, 537-540),
+// projection outputs -> f16 (tensor.rs:1623-1643), K and V -> f16 on cache write (transformer.rs:754-761),
+// attention output -> f16 (transformer.rs:793-796), SiLU*gate -> f16 (transformer.rs:563-565).  The reference
+// keeps q (after RoPE) and the softmax probabilities in fp32; to feed them to the f16 matrix cores without
+// losing that, each is split into a high and a low f16 part (v = hi + lo to about 2^-22 relative) and the
+// product is accumulated over both parts.
+#include "kernels.h"
+#include "device_utils.h"
+
+namespace rlh {
+
+// X[r, :] = table[tokens[r], :] widened to f32 (embedding.rs:50-52, transformer.rs:361-367)
+template <typename ET>
+__global__ void embed_rows_kernel(const ET *table, const int32_t *tokens, int dim, float *x) {
+    const int r = blockIdx.x;
+    const size_t tok = (size_t)tokens[r];
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) x[(size_t)r * dim + i] = (float)table[tok * dim + i];
+}
+
+hipError_t launch_embed_rows(const void *table, int table_f16, const int32_t *tokens_dev, int n, int dim, float *x, hipStream_t s) {
+    if (table_f16) hipLaunchKernelGGL(embed_rows_kernel<half_t>, dim3(n), dim3(256), 0, s, (const half_t *)table, tokens_dev, dim, x);
+    else hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(n), dim3(256), 0, s, (const float *)table, tokens_dev, dim, x);
+    return hipGetLastError();
+}
+
+// RMSNorm::forward per row (transformer.rs:476-480), output rounded to f16 for the projections that follow
+__global__ __launch_bounds__(256) void rmsnorm_rows_f16_kernel(half_t *y, const float *x, const float *w, int d, float eps) {
+    __shared__ float red[16];
+    const float *xr = x + (size_t)blockIdx.x * d;
+    half_t *yr = y + (size_t)blockIdx.x * d;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
+    ss = block_sum(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) yr[i] = (half_t)((xr[i] * rs) * w[i]);
+}
+
+hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s) {
+    hipLaunchKernelGGL(rmsnorm_rows_f16_kernel, dim3(rows), dim3(256), 0, s, (half_t *)y, x, w, d, eps);
+    return hipGetLastError();
+}
+
+// qkv [n x 3 dim] f16 (rows = tokens at positions 0..n-1) ->
+//   q after RoPE, split hi/lo, head-major [head][n][head_dim]
+//   K (after RoPE) and V into the cache [head][max_seq_len][head_dim] at positions 0..n-1
+//   V transposed [head][head_dim][t_pad] (positions contiguous) as the B operand of P.V
+__global__ void rope_kv_prefill_kernel(PrefillRopeParams p) {
+    const int half_hd = p.head_dim / 2;
+    const int pairs_per_row = p.dim / 2;
+    const size_t total = (size_t)p.n * pairs_per_row;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const half_t *qkv = reinterpret_cast<const half_t *>(p.qkv);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int r = (int)(i / pairs_per_row);              // token row = position
+        const int pr = (int)(i - (size_t)r * pairs_per_row); // pair within the row
+        const int head = pr / half_hd, c = pr - head * half_hd;
+        const int j = head * p.head_dim + 2 * c;
+        const float2 f = p.freqs[(size_t)r * half_hd + c];
+        const half_t *row = qkv + (size_t)r * 3 * p.dim;
+        // q
+        float a, b;
+        rope_pair((float)row[j], (float)row[j + 1], f, a, b);
+        const size_t qo = ((size_t)head * p.n + r) * p.head_dim + 2 * c;
+        half_t *qhi = reinterpret_cast<half_t *>(p.q_hi), *qlo = reinterpret_cast<half_t *>(p.q_lo);
+        const half_t ah = (half_t)a, bh = (half_t)b;
+        qhi[qo] = ah;
+        qhi[qo + 1] = bh;
+        qlo[qo] = (half_t)(a - (float)ah);
+        qlo[qo + 1] = (half_t)(b - (float)bh);
+        // k
+        rope_pair((float)row[p.dim + j], (float)row[p.dim + j + 1], f, a, b);
+        const size_t co = ((size_t)head * p.max_seq_len + r) * p.head_dim + 2 * c;
+        const float v0 = (float)row[2 * p.dim + j], v1 = (float)row[2 * p.dim + j + 1];
+        if (p.cache_f16) {
+            half_t *ck = reinterpret_cast<half_t *>(p.cache_k), *cv = reinterpret_cast<half_t *>(p.cache_v);
+            ck[co] = (half_t)a; // Tensor::set_f32 on an f16 cache (tensor.rs:373-376)
+            ck[co + 1] = (half_t)b;
+            cv[co] = (half_t)v0;
+            cv[co + 1] = (half_t)v1;
+        } else {
+            float *ck = reinterpret_cast<float *>(p.cache_k), *cv = reinterpret_cast<float *>(p.cache_v);
+            ck[co] = a;
+            ck[co + 1] = b;
+            cv[co] = v0;
+            cv[co + 1] = v1;
+        }
+        half_t *vt = reinterpret_cast<half_t *>(p.v_t);
+        vt[((size_t)head * p.head_dim + 2 * c) * p.t_pad + r] = (half_t)v0;
+        vt[((size_t)head * p.head_dim + 2 * c + 1) * p.t_pad + r] = (half_t)v1;
+    }
+}
+
+hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s) {
+    const size_t total = (size_t)p.n * (p.dim / 2);
+    const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+    hipLaunchKernelGGL(rope_kv_prefill_kernel, dim3(blocks), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
+// Scores [head][n][t_pad] f32 (raw q.k) -> causal softmax probabilities split hi/lo f16 [head][n][t_pad].
+// scalar_multiply_f32(1/sqrt(hd)), + full_triu mask, softmax (transformer.rs:768-779; tensor.rs:496-508, 479-494);
+// evaluated with the row maximum subtracted, which is the same function wherever the reference's is finite.
+// One wavefront per row; masked and padded columns get probability 0.
+__global__ __launch_bounds__(256) void causal_softmax_kernel(const float *scores, half_t *p_hi, half_t *p_lo, size_t total_rows, int n, int t_pad,
+                                                             float scale) {
+    const int lane = threadIdx.x & 63;
+    const size_t row_id = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6); // over heads * n
+    if (row_id >= total_rows) return;                                  // whole wavefronts leave together
+    const int r = (int)(row_id % (size_t)n);                           // row r attends to columns 0..r
+    const float *srow = scores + row_id * t_pad;
+    half_t *hi = p_hi + row_id * t_pad;
+    half_t *lo = p_lo + row_id * t_pad;
+    float mx = -INFINITY;
+    for (int c = lane; c <= r; c += 64) mx = fmaxf(mx, srow[c] * scale);
+    mx = wave_max(mx);
+    float sum = 0.0f;
+    for (int c = lane; c <= r; c += 64) sum += expf(srow[c] * scale - mx);
+    sum = wave_sum(sum);
+    for (int c = lane; c < t_pad; c += 64) {
+        float pv = 0.0f;
+        if (c <= r) pv = expf(srow[c] * scale - mx) / sum;
+        const half_t h = (half_t)pv;
+        hi[c] = h;
+        lo[c] = (half_t)(pv - (float)h);
+    }
+}
+
+hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int head_dim, hipStream_t s) {
+    const size_t rows = (size_t)n_heads * n;
+    hipLaunchKernelGGL(causal_softmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, scores, (half_t *)p_hi, (half_t *)p_lo, rows, n, t_pad,
+                       1.0f / sqrtf((float)head_dim)); // transformer.rs:770
+    return hipGetLastError();
+}
+
+// attention output [head][n][head_dim] f32 -> [n][dim] f16: the concat of heads per row and the f16 rounding
+// point before wo (transformer.rs:783-796)
+__global__ void attn_out_f16_kernel(const float *o, half_t *a, int n, int n_heads, int head_dim) {
+    const size_t total = (size_t)n * n_heads * head_dim;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const int dim = n_heads * head_dim;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int r = (int)(i / dim);
+        const int j = (int)(i - (size_t)r * dim);
+        const int head = j / head_dim, jj = j - head * head_dim;
+        a[i] = (half_t)o[((size_t)head * n + r) * head_dim + jj];
+    }
+}
+
+hipError_t launch_attn_out_f16(const float *o, void *a, int n, int n_heads, int head_dim, hipStream_t s) {
+    const size_t total = (size_t)n * n_heads * head_dim;
+    const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+    hipLaunchKernelGGL(attn_out_f16_kernel, dim3(blocks), dim3(256), 0, s, o, (half_t *)a, n, n_heads, head_dim);
+    return hipGetLastError();
+}
+
+// m = f16r(silu(g) * u) on f16 tensors (transformer.rs:557-565; tensor.rs:822-832, 722-734)
+__global__ void silu_mul_f16_kernel(const half_t *g, const half_t *u, half_t *m, size_t total) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const float gv = (float)g[i];
+        const float sg = gv / (1.0f + expf(-gv));
+        m[i] = (half_t)(sg * (float)u[i]);
+    }
+}
+
+hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s) {
+    const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+    hipLaunchKernelGGL(silu_mul_f16_kernel, dim3(blocks), dim3(256), 0, s, (const half_t *)g, (const half_t *)u, (half_t *)m, total);
+    return hipGetLastError();
+}
+
+} // namespace rlh

@@ -327,3 +327,45 @@ def test_percentage_to_gpu_rule(ctx):
                                    shape.max_seq_len, shape.norm_eps, ds)
         assert m.last_layer_on_gpu() == want, p
         m.free()
+
+
+@pytest.mark.parametrize("n,m_rows,k", [(2, 3, 8), (33, 65, 72), (128, 128, 64), (130, 200, 192), (16, 2816, 1024), (257, 384, 4096), (1024, 256, 11008)])
+def test_mfma_gemm_f16(ctx, n, m_rows, k):
+    """src [n x k] . other[m x k]^T with n > 1 runs on the matrix cores; every element against the oracle's
+    f16-rounded dot8 (tensor.rs:1476-1666), including tiles that straddle the matrix edges."""
+    rng = np.random.default_rng(n * 7 + m_rows * 3 + k)
+    a = oracle.f32_to_f16_bits(rng.uniform(-1, 1, (n, k)).astype(f32))
+    b = oracle.f32_to_f16_bits((rng.standard_normal((m_rows, k)) * 0.05).astype(f32))
+    got = Tensor.from_numpy(ctx, a).matrix_mul_transposed(Tensor.from_numpy(ctx, b)).to_numpy().astype(f32)
+    want = oracle.f16_bits_to_f32(oracle.matmul_transposed_f16(a, b))
+    mag = np.abs(oracle.f16_bits_to_f32(a).astype(np.float64)) @ np.abs(oracle.f16_bits_to_f32(b).astype(np.float64)).T
+    close_f16(got, want, mag, f"mfma gemm {n}x{m_rows}x{k}")
+    assert np.mean(got != want) < 0.03
+
+
+def test_prefill_matrix_core_path_against_token_by_token_and_oracle(ctx):
+    """n > 1 at start_pos 0 in f16 mode: the matrix-core prefill and the token-by-token path are the same function
+    (transformer.rs:343-383); both stay within tolerance of the oracle's prefill, and leave the same KV cache."""
+    shape = Shape(dim=256, n_layers=3, n_heads=4, ffn_hidden=704, vocab_size=512, max_seq_len=200)
+    W = synth_weights(shape, seed=41, std=0.08, norm_ones=False)
+    toks = np.random.default_rng(42).integers(0, shape.vocab_size, 150)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    for n in (2, 33, 129, 150):
+        want = om.forward(toks[:n], 0, om.make_caches())
+        ga, gb = gm.make_caches(), gm.make_caches()
+        gm.set_prefill_mode(False)
+        a = gm.forward(toks[:n], 0, ga)
+        gm.set_prefill_mode(True)
+        b = gm.forward(toks[:n], 0, gb)
+        gm.set_prefill_mode(False)
+        assert max_rel_err(a, want) < TOL_F16 and max_rel_err(b, want) < TOL_F16, (n, max_rel_err(a, want), max_rel_err(b, want))
+        assert max_rel_err(a, b) < TOL_F16
+        for l in (0, shape.n_layers - 1):
+            for which in (0, 1):
+                ca, cb = ga.read(l, 1, which), gb.read(l, 1, which)
+                assert not np.any(ca[:, n:]) and not np.any(cb[:, n:])
+                assert np.all(np.abs(ca[:, :n] - cb[:, :n]) <= 2 * ulp_f16(cb[:, :n]) + 2e-3 * np.abs(cb[:, :n]).max())
+        # decode continues from a matrix-core prefill exactly as from a token-by-token one
+        nxt = int(toks[n % len(toks)])
+        assert max_rel_err(gm.forward([nxt], n, ga), gm.forward([nxt], n, gb)) < TOL_F16
+    gm.free()
