@@ -30,6 +30,7 @@ CONFIGS = {
     "c0": (1024, 8, 16, 2816, 32000, 16, 64),
     "c1": (4096, 32, 32, 11008, 32000, 128, 256),
     "c2": (5120, 40, 40, 13824, 32000, 2048, 128),
+    "c3": (4096, 32, 32, 11008, 32000, 1024, 1),          # prompt prefill: one forward over 1024 tokens
     "c4": (8192, 80, 64, 22016, 32000, 256, 128),
 }
 
@@ -127,6 +128,41 @@ def main() -> int:
     model = ra.Transformer(ctx, dim, n_layers, n_heads, ffn, vocab, max_seq, 1e-6, ds)
     model.fill_synthetic(seed=0, std=0.02)
     prompt = ra.synth_tokens(0, n_prompt, 3, vocab)
+
+    if args.config == "c3":
+        # prefill: time-to-first-token of one n_prompt-token forward (+ greedy pick), TFLOP/s against the dense f16 MFMA peak
+        reps = max(1, K)
+        model.generate_greedy(prompt, 1, model.make_caches())            # warm-up (also sizes the work buffers)
+        times = []
+        for _ in range(reps):
+            cc = model.make_caches()
+            ctx.sync()
+            t0 = time.perf_counter()
+            _, ms_first, _ = model.generate_greedy(prompt, 1, cc)
+            ctx.sync()
+            times.append((1e3 * (time.perf_counter() - t0), ms_first))
+            cc.free()
+        wall_ms = float(np.mean([t[0] for t in times]))
+        ev_ms = float(np.mean([t[1] for t in times]))
+        n = n_prompt
+        flops_linear = 2.0 * n * n_layers * (4 * dim * dim + 3 * dim * ffn)
+        flops_attn = 2.0 * n * n * dim * n_layers          # causal: half of the dense 4 n^2 d
+        flops_head = 2.0 * vocab * dim
+        tflops = (flops_linear + flops_attn + flops_head) / (ev_ms * 1e-3) / 1e12
+        out = {
+            "metric": "time to first token, LLaMA-7B-shape f16 prompt prefill (1024 tokens), 1 MI355X",
+            "value": round(wall_ms, 3), "unit": "ms", "n_gpus": 1, "steps": reps, "warmup": 1, "ms_per_step": round(wall_ms, 3),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, fp32 accumulate (MFMA)",
+            "data": "synthetic (random-init N(0,0.02) weights seed 0, synthetic token ids)",
+            "config": {"workload": f"c3: dim {dim}, {n_layers} layers, {n_heads} heads, ffn {ffn}; one forward over {n} prompt tokens"},
+            "ms_hip_events": round(ev_ms, 3), "tokens_per_s": round(n / (wall_ms * 1e-3), 1),
+            "roofline": {"bound": "mfma", "kernel": "gemm_f16_kernel (128x128x64 tiles, v_mfma_f32_32x32x16_f16)", "achieved": round(tflops, 1),
+                         "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tflops / 2500.0, 4), "traffic": None,
+                         "algorithmic_flops": flops_linear + flops_attn + flops_head},
+            "cpu_baseline": None, "device": info["name"],
+        }
+        print(json.dumps(out))
+        return 0
 
     if args.kernels_only:
         caches = model.make_caches()
