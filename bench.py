@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+# HBM bytes per launch of the dominant decode kernel (w13 GEMV, 7B shape) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs, each scaled by the same counter on a 1 GiB copy kernel (the PMC summary under profiles/ has the commands).
+MEASURED_TRAFFIC = {"c1": 180_960_678}
 
 CONFIGS = {
     # name: (dim, n_layers, n_heads, ffn_hidden, vocab, n_prompt, default decode steps)
@@ -207,7 +210,7 @@ def main() -> int:
     roofline = {
         "bound": "hbm", "kernel": "gemv_kernel<f16 weights, f16 x, SiLU epilogue> (" + dom + ")",
         "achieved": kernels[dom]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": round(kernels[dom]["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+        "frac": round(kernels[dom]["GBps"] / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC.get(args.config),
         "algorithmic_bytes_per_launch": kernels[dom]["bytes"], "us_per_launch": kernels[dom]["us"],
     }
 

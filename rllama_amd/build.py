@@ -70,5 +70,22 @@ def build(force: bool = False) -> str:
     return LIB
 
 
+HOST_BIN = os.path.join(HERE, "host", "rllama_generate")
+
+
+def build_host(force: bool = False) -> str:
+    """Compiles the C++ host example (header-only mirror of the reference API + the token loop) against the library."""
+    src = os.path.join(HERE, "host", "generate_main.cpp")
+    hdr = os.path.join(HERE, "host", "rllama_hip.hpp")
+    if not force and os.path.exists(HOST_BIN) and all(os.path.getmtime(HOST_BIN) >= os.path.getmtime(f) for f in (src, hdr, LIB)):
+        return HOST_BIN
+    cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-Wextra", src, "-o", HOST_BIN, "-L" + HERE, "-lrllama_hip", "-Wl,-rpath,$ORIGIN/.."]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("host build failed:\n" + " ".join(cmd) + "\n" + r.stdout + r.stderr)
+    return HOST_BIN
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv))
+    print(build_host(force="--force" in sys.argv))
