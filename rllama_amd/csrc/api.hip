@@ -13,6 +13,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -106,7 +107,9 @@ struct rlh_model {
     int32_t *prompt_dev = nullptr;
     int prompt_cap = 0;
     float *attn_ws = nullptr;
-    int max_splits = 16;
+    int max_splits = 32;
+    int attn_single_max = 256; // sequence lengths up to this use one block per head
+    int attn_chunk = 128;      // positions per block beyond that
     int stream_weights = 1;
     PrefillScratch pf;
     int prefill_mode = 0; // 0: matrix-core prefill where available (f16 mode), 1: token by token
@@ -256,6 +259,14 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     m->prm = *prm;
     m->prm.percentage_to_gpu = clamp_percentage(prm->percentage_to_gpu);
     m->head_dim = hd;
+    if (const char *e = getenv("RLLAMA_HIP_ATTN_CHUNK")) { // tuning knobs: positions per attention block / single-block limit
+        const int v = atoi(e);
+        if (v >= 16) m->attn_chunk = v;
+    }
+    if (const char *e = getenv("RLLAMA_HIP_ATTN_SINGLE_MAX")) {
+        const int v = atoi(e);
+        if (v >= 0) m->attn_single_max = v;
+    }
     // transformer.rs:266-268
     m->last_layer_on_gpu = (int)std::round(m->prm.percentage_to_gpu * (float)(prm->n_layers - 1));
     m->layers.resize((size_t)prm->n_layers);
@@ -615,9 +626,10 @@ extern "C" int rlh_caches_read(const rlh_caches *c, int layer, int head, int whi
 // forward
 // ------------------------------------------------------------------------------------------------
 static int attn_splits(const rlh_model *m, int T) {
-    // One block per (head, split).  A block streams its share of the cache alone, so short sequences stay
-    // in one block per head; longer ones are cut into chunks of about 256 positions.
-    int S = (T + 255) / 256;
+    // One block per (head, split).  A block streams its share of the cache alone, so short sequences stay in one
+    // block per head (no merge launch); longer ones are cut into chunks of about attn_chunk positions.
+    if (T <= m->attn_single_max) return 1;
+    int S = (T + m->attn_chunk - 1) / m->attn_chunk;
     if (S < 1) S = 1;
     if (S > m->max_splits) S = m->max_splits;
     return S;

@@ -6,8 +6,8 @@
 //
 // Here the cache is laid out [head][position][head_dim], so that one position's K (or V) row is contiguous:
 // a lane owns 8 consecutive dims, head_dim / 8 lanes make one position, and a wave covers 64 / (head_dim / 8)
-// positions per step with 16-byte loads.  K and V rows of a step are loaded together and the next step's
-// rows are already in flight while the current ones are consumed.  Every lane group keeps a running
+// positions per step with 16-byte loads.  K and V rows of several steps are loaded together before any is
+// consumed (independent loads in flight hide the memory latency; a single query leaves nothing to reuse).  Every lane group keeps a running
 // (max, sum, weighted V) triple (the max-subtracted form equals the reference's exp(s) / sum exp(s)
 // wherever that is finite), so the main loop has no block-wide synchronisation; the groups' triples are
 // merged once at the end through LDS.  Long sequences are split over several blocks per head
@@ -17,8 +17,15 @@
 
 namespace rlh {
 
-constexpr int kAttnThreads = 512;
+#ifndef RLH_ATTN_THREADS
+#define RLH_ATTN_THREADS 512
+#endif
+#ifndef RLH_ATTN_BATCH
+#define RLH_ATTN_BATCH 4
+#endif
+constexpr int kAttnThreads = RLH_ATTN_THREADS;
 constexpr int kAttnWaves = kAttnThreads / kWave;
+constexpr int kAttnBatch = RLH_ATTN_BATCH; // cache rows of K and of V loaded together per lane
 
 template <typename CT>
 __device__ __forceinline__ void load8(const CT *p, float (&out)[8]) {
@@ -37,8 +44,27 @@ __device__ __forceinline__ void load8(const CT *p, float (&out)[8]) {
     }
 }
 
+// 8 consecutive cache elements of one lane: one 16-byte word (f16) or two (f32)
+template <typename CT>
+__device__ __forceinline__ void unpack8(const uint4_t *raw, float (&out)[8]) {
+    if constexpr (sizeof(CT) == 2) {
+        half8_t h = __builtin_bit_cast(half8_t, raw[0]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) out[i] = (float)h[i];
+    } else {
+        float4_t a = __builtin_bit_cast(float4_t, raw[0]);
+        float4_t b = __builtin_bit_cast(float4_t, raw[1]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            out[i] = a[i];
+            out[i + 4] = b[i];
+        }
+    }
+}
+
 template <typename CT, int kHeadDim>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeParams p) {
+    constexpr int kRawPerRow = sizeof(CT) == 2 ? 1 : 2;
     constexpr int kLanesPerPos = kHeadDim / 8;        // each lane owns 8 consecutive dims
     constexpr int kPosPerWave = kWave / kLanesPerPos; // positions per wave step
     constexpr int kSets = kAttnWaves * kPosPerWave;   // lane groups in the block, one partial triple each
@@ -75,34 +101,40 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
     for (int i = 0; i < 8; i++) acc[i] = 0.0f;
 
     // this lane group's positions: t0 + (wave + g * kAttnWaves) * kPosPerWave + sub, g = 0, 1, ...
+    // kAttnBatch steps are loaded together (2 * kAttnBatch independent 16-byte loads in flight per lane)
     const int stride = kAttnWaves * kPosPerWave;
-    int t = t0 + wave * kPosPerWave + sub;
-    float kc[8], vc[8], kn[8], vn[8];
     const int t_safe = t1 > t0 ? t1 - 1 : 0; // address clamp for lanes past the end (their values are discarded)
-    load8<CT>(kbase + (size_t)min(t, t_safe) * kHeadDim, kc);
-    load8<CT>(vbase + (size_t)min(t, t_safe) * kHeadDim, vc);
-    // the loop bound is wave-uniform: the wave's first position decides, lanes past t1 are masked by `valid`
-    for (int tw = t0 + wave * kPosPerWave; tw < t1; tw += stride, t += stride) {
-        const int tn = t + stride;
-        load8<CT>(kbase + (size_t)min(tn, t_safe) * kHeadDim, kn);
-        load8<CT>(vbase + (size_t)min(tn, t_safe) * kHeadDim, vn);
-        float part = 0.0f;
+    int t = t0 + wave * kPosPerWave + sub;
+    // the loop bound is wave-uniform: the wave's first position decides, lanes past t1 are masked
+    for (int tw = t0 + wave * kPosPerWave; tw < t1; tw += stride * kAttnBatch, t += stride * kAttnBatch) {
+        uint4_t kraw[kAttnBatch][kRawPerRow], vraw[kAttnBatch][kRawPerRow];
 #pragma unroll
-        for (int i = 0; i < 8; i++) part = fmaf(qv[i], kc[i], part);
-        const float s = group_sum<kLanesPerPos>(part) * scale;
-        if (t < t1) {
-            const float m_new = fmaxf(m_run, s);
-            const float alpha = expf(m_run - m_new);
-            const float pe = expf(s - m_new);
-            l_run = fmaf(l_run, alpha, pe);
+        for (int u = 0; u < kAttnBatch; u++) {
+            const size_t off = (size_t)min(t + u * stride, t_safe) * kHeadDim;
 #pragma unroll
-            for (int i = 0; i < 8; i++) acc[i] = fmaf(acc[i], alpha, pe * vc[i]);
-            m_run = m_new;
+            for (int w = 0; w < kRawPerRow; w++) {
+                kraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(kbase + off) + 16 * w);
+                vraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(vbase + off) + 16 * w);
+            }
         }
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            kc[i] = kn[i];
-            vc[i] = vn[i];
+        for (int u = 0; u < kAttnBatch; u++) {
+            float kc[8], vc[8];
+            unpack8<CT>(kraw[u], kc);
+            unpack8<CT>(vraw[u], vc);
+            float part = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) part = fmaf(qv[i], kc[i], part);
+            const float s = group_sum<kLanesPerPos>(part) * scale;
+            if (t + u * stride < t1) {
+                const float m_new = fmaxf(m_run, s);
+                const float alpha = expf(m_run - m_new);
+                const float pe = expf(s - m_new);
+                l_run = fmaf(l_run, alpha, pe);
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[i] = fmaf(acc[i], alpha, pe * vc[i]);
+                m_run = m_new;
+            }
         }
     }
 
@@ -139,23 +171,46 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
     }
 }
 
-// Merges the per-split triples of one head: grid = heads, block = head_dim threads.
+// Merges the per-split triples of one head: grid = heads, block = max(head_dim, 64) threads.  The first wavefront
+// turns the (max, sum) pairs into one weight per split (one load per lane, wave reductions); then thread j sums
+// the weighted partial outputs of dim j with independent loads.
+constexpr int kAttnMaxSplits = 64;
 __global__ void attn_merge_kernel(const float *workspace, int n_splits, int head_dim, float *out, int round_out) {
+    __shared__ float wgt[kAttnMaxSplits];
+    __shared__ float l_total;
     const int head = blockIdx.x;
-    const int j = threadIdx.x;
+    const int tid = threadIdx.x;
     const float *wh = workspace + (size_t)head * n_splits * (head_dim + 2);
-    float M = -INFINITY;
-    for (int s = 0; s < n_splits; s++) M = fmaxf(M, wh[(size_t)s * (head_dim + 2)]);
-    float L = 0.0f, O = 0.0f;
-    for (int s = 0; s < n_splits; s++) {
-        const float *w = wh + (size_t)s * (head_dim + 2);
-        const float ls = w[1];
-        const float f = ls > 0.0f ? expf(w[0] - M) : 0.0f;
-        L = fmaf(ls, f, L);
-        O = fmaf(w[2 + j], f, O);
+    if (tid < kWave) {
+        float ms = -INFINITY, ls = 0.0f;
+        if (tid < n_splits) {
+            ms = wh[(size_t)tid * (head_dim + 2)];
+            ls = wh[(size_t)tid * (head_dim + 2) + 1];
+        }
+        const float M = wave_max(ms);
+        const float f = ls > 0.0f ? expf(ms - M) : 0.0f;
+        const float L = wave_sum(ls * f);
+        if (tid < n_splits) wgt[tid] = f;
+        if (tid == 0) l_total = L;
     }
-    const float o = O / L;
-    out[head * head_dim + j] = round_out ? f16r(o) : o;
+    __syncthreads();
+    if (tid < head_dim) {
+        float O = 0.0f;
+        int s = 0;
+        for (; s + 4 <= n_splits; s += 4) {
+            const float o0 = wh[(size_t)(s + 0) * (head_dim + 2) + 2 + tid];
+            const float o1 = wh[(size_t)(s + 1) * (head_dim + 2) + 2 + tid];
+            const float o2 = wh[(size_t)(s + 2) * (head_dim + 2) + 2 + tid];
+            const float o3 = wh[(size_t)(s + 3) * (head_dim + 2) + 2 + tid];
+            O = fmaf(o0, wgt[s], O);
+            O = fmaf(o1, wgt[s + 1], O);
+            O = fmaf(o2, wgt[s + 2], O);
+            O = fmaf(o3, wgt[s + 3], O);
+        }
+        for (; s < n_splits; s++) O = fmaf(wh[(size_t)s * (head_dim + 2) + 2 + tid], wgt[s], O);
+        const float o = O / l_total;
+        out[head * head_dim + tid] = round_out ? f16r(o) : o;
+    }
 }
 
 template <typename CT>
@@ -172,11 +227,12 @@ static hipError_t launch_attn_t(const AttnDecodeParams &p, hipStream_t s) {
 }
 
 hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s) {
-    if (p.n_splits < 1) return hipErrorInvalidValue;
+    if (p.n_splits < 1 || p.n_splits > kAttnMaxSplits) return hipErrorInvalidValue;
     if (p.n_splits > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
     hipError_t e = p.cache_f16 ? launch_attn_t<half_t>(p, s) : launch_attn_t<float>(p, s);
     if (e != hipSuccess || p.n_splits == 1) return e;
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(p.n_heads), dim3(p.head_dim), 0, s, p.workspace, p.n_splits, p.head_dim, p.out, p.round_out);
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(p.n_heads), dim3(p.head_dim < kWave ? kWave : p.head_dim), 0, s, p.workspace, p.n_splits, p.head_dim, p.out,
+                       p.round_out);
     return hipGetLastError();
 }
 
