@@ -77,7 +77,7 @@ struct Layer {
 // Work buffers of a multi-token forward (prefill); grown on demand, kept for the next call.
 struct PrefillScratch {
     int n_cap = 0;       // rows the buffers are sized for
-    int t_pad = 0;       // n_cap rounded up to 8: row stride of scores / probabilities / transposed V
+    int t_pad = 0;       // n_cap rounded up to 64: row stride of scores / probabilities / transposed V
     float *x = nullptr, *h = nullptr, *scores = nullptr, *o = nullptr;
     void *xn = nullptr, *qkv = nullptr, *q_hi = nullptr, *q_lo = nullptr, *v_t = nullptr, *p_hi = nullptr, *p_lo = nullptr, *a = nullptr;
     void *g = nullptr, *u = nullptr, *mm = nullptr;
@@ -783,7 +783,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     if (n <= S.n_cap) return RLH_OK;
     S.release();
     const size_t d = (size_t)m->prm.dim, F = (size_t)m->prm.ffn_hidden, H = (size_t)m->prm.n_heads, hd = (size_t)m->head_dim;
-    const size_t N = (size_t)n, tp = (N + 7) & ~(size_t)7;
+    const size_t N = (size_t)n, tp = (N + 63) & ~(size_t)63;
     hipError_t e = hipSuccess;
     auto A = [&](void **p, size_t bytes) {
         if (e != hipSuccess) return;
@@ -825,7 +825,7 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     const rlh_model_params &P = m->prm;
     PrefillScratch &S = m->pf;
     const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size, H = P.n_heads, hd = m->head_dim;
-    const int tp = (n + 7) & ~7; // row stride of this call's scores / probabilities / transposed V
+    const int tp = (n + 63) & ~63; // row stride of this call's scores / probabilities / transposed V (a whole number of K-tiles)
     const float eps = (float)P.norm_eps;
     HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
     HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));

@@ -16,6 +16,8 @@
 #include "kernels.h"
 #include "device_utils.h"
 
+#include <cstdlib>
+
 namespace rlh {
 
 constexpr int kBM = 128, kBN = 128, kBK = 64;
@@ -126,6 +128,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_f16_kernel(GemmParams p) {
 
 hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s) {
     if (p.m <= 0 || p.n <= 0 || p.k <= 0 || (p.k % 8) != 0 || (p.lda % 8) != 0 || (p.ldb % 8) != 0 || p.batch < 1) return hipErrorInvalidValue;
+    // RLLAMA_HIP_GEMM_SIMPLE=1 keeps every product on the kernel of this file (tuning / cross-checks)
+    static const bool simple_only = getenv("RLLAMA_HIP_GEMM_SIMPLE") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_SIMPLE")) != 0;
+    if (!simple_only && gemm_f16_dma_supported(p)) return launch_gemm_f16_dma(p, epilogue, s);
     dim3 grid((p.n + kBN - 1) / kBN, (p.m + kBM - 1) / kBM, p.batch);
     switch (epilogue) {
     case kGemmEpiF16: hipLaunchKernelGGL(gemm_f16_kernel<kGemmEpiF16>, grid, dim3(kGemmThreads), 0, s, p); break;
