@@ -1,116 +1,171 @@
 // gemm_dma.hip -- the fast path of the prefill GEMM  C = A * B^T  (f16 operands, fp32 accumulate) on gfx950.
 //
-// Same contract as gemm.hip's kernel, restricted to K % 64 == 0.  What differs is how operands reach LDS:
+// Same contract as gemm.hip's kernel, restricted to K % 32 == 0.  What differs is how operands reach LDS and how
+// large a tile a workgroup owns:
 //   * direct global -> LDS loads (global_load_lds_dwordx4: each lane names a global address, the 64 x 16 bytes
 //     of a wavefront land contiguously in LDS), so no registers and no ds_write are spent on staging and a
-//     load can stay in flight for several K-tiles: four LDS stages, the loads of K-tile t + 2 are issued while
-//     K-tile t feeds the matrix cores, one barrier per K-tile;
-//   * LDS rows are 128 bytes (64 halves) without padding; the 16-byte chunk c of row r is stored at chunk
-//     c ^ ((r >> 1) & 7), which makes the MFMA operand reads (16 consecutive rows, same logical chunk) hit 16
-//     distinct bank groups, and is free on the store side because every lane chooses its own global address.
-// Workgroup tile 128 x 128, 4 wavefronts of 64 x 64 (2 x 2 v_mfma_f32_32x32x16_f16).
+//     load can stay in flight across K-tiles: several LDS stages, the loads of K-tile t + stages - 1 are issued
+//     while K-tile t feeds the matrix cores, one barrier per K-tile;
+//   * LDS rows are 2 kBK bytes without padding; the 16-byte chunk c of row r is stored at a chunk XOR-ed
+//     with a function of r, which makes the MFMA operand reads (16 consecutive rows, same logical chunk) hit 16
+//     distinct bank groups, and is free on the store side because every lane chooses its own global address;
+//   * the tile is a template parameter.  What bounds this kernel is the L2 -> LDS traffic, which falls with the
+//     tile edge: 128 x 128 moves 1 byte per 64 flop, 256 x 256 one per 128 flop.  launch_gemm_f16_dma picks the
+//     tile by a small cost model (rounds of workgroups over the compute units x tile efficiency).
+// Wavefronts form a (kWavesM x 2) grid; each owns 64 x (32 kNT) of C = 2 x kNT v_mfma_f32_32x32x16_f16 tiles.
 #include "kernels.h"
 #include "device_utils.h"
 
+#include <cstdlib>
+
 namespace rlh {
 
-constexpr int kDmaBM = 128, kDmaBN = 128, kDmaBK = 64;
-constexpr int kDmaStages = 4;
-constexpr int kDmaThreads = 256;
-constexpr int kDmaStageBytes = (kDmaBM + kDmaBN) * kDmaBK * 2; // 32 KiB
-constexpr int kDmaLoadsPerWave = (kDmaBM + kDmaBN) / 8 / 4;    // 1 KiB loads (8 rows) per wavefront and K-tile
+constexpr int kDmaMinBK = 32;
 
 typedef __attribute__((ext_vector_type(16))) float float16_t;
 
-template <int kEpi>
-__global__ __launch_bounds__(kDmaThreads) void gemm_f16_dma_kernel(GemmParams p) {
+// One direct-to-LDS load: lane l's 16 bytes at `src` land at LDS byte address dst + 16 l (dst is wave-uniform and
+// travels in M0).  Written as inline assembly on purpose: through the builtin the compiler tracks the load as an LDS
+// write and puts s_waitcnt vmcnt(0) in front of every LDS read, which would also wait for the prefetched K-tiles;
+// here the waits are placed by hand (vmcnt is decremented in issue order).
+__device__ __forceinline__ void dma16(const half_t *src, unsigned dst) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory");
+}
+
+template <int kN>
+__device__ __forceinline__ void wait_vmcnt() { // s_waitcnt vmcnt(kN) only (6-bit count: bits 3:0 and 15:14)
+    static_assert(kN >= 0 && kN < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kN & 0xF) | ((kN >> 4) << 14));
+}
+
+// kWavesM: wavefront rows (tile height 64 kWavesM); kNT: 32-column MFMA tiles per wavefront (tile width 64 kNT);
+// kBK: halves of K per tile (32 or 64); kStages: LDS stages (K-tiles in flight).
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages>
+__global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams p) {
+    constexpr int kWaves = 2 * kWavesM;
+    constexpr int kBM = 64 * kWavesM, kBN = 64 * kNT;
+    constexpr int kCpr = kBK / 8;                        // 16-byte chunks per LDS row
+    constexpr int kRowsPerLoad = 64 / kCpr;              // rows one wavefront-wide load covers (1 KiB of LDS)
+    constexpr int kSwzDiv = 16 / kCpr;                   // physical chunk = logical chunk ^ ((row / kSwzDiv) % kCpr)
+    constexpr int kRowBytes = kBK * 2;
+    constexpr int kStageBytes = (kBM + kBN) * kRowBytes;
+    constexpr int kGroups = kStageBytes / 1024;          // 1 KiB row groups per stage, dealt round-robin to wavefronts
+    constexpr int kLoadsMax = (kGroups + kWaves - 1) / kWaves;
+    constexpr int kLoadsMin = kGroups / kWaves;
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int bm0 = blockIdx.y * kDmaBM, bn0 = blockIdx.x * kDmaBN;
+    const int bm0 = blockIdx.y * kBM, bn0 = blockIdx.x * kBN;
     const size_t zb = blockIdx.z;
     const half_t *A = p.a + zb * p.stride_a;
     const half_t *B = p.b + zb * p.stride_b;
     const int M = p.m, N = p.n, K = p.k;
-    const int n_kt = K / kDmaBK;
+    const int n_kt = K / kBK;
 
-    // ---- staging: wavefront w moves row groups (8 rows = 1 KiB of LDS) w*8 .. w*8+7 of the 32 groups of a stage
-    //      (groups 0..15 = A rows, 16..31 = B rows).  Lane i of a group: row i / 8, physical chunk i % 8.
-    const int l_row = lane >> 3, l_pc = lane & 7;
-    const half_t *gsrc[kDmaLoadsPerWave];
+    // ---- staging: a stage holds rows 0 .. kBM-1 of A then rows 0 .. kBN-1 of B, kRowBytes each.  Load i of
+    //      wavefront w moves row group i * kWaves + w; lane l of a group: row l / kCpr, physical chunk l % kCpr.
+    const int l_row = lane / kCpr, l_pc = lane % kCpr;
+    const bool short_wave = kLoadsMax != kLoadsMin && (kLoadsMax - 1) * kWaves + wave >= kGroups; // one load fewer
+    const half_t *gsrc[kLoadsMax];
 #pragma unroll
-    for (int i = 0; i < kDmaLoadsPerWave; i++) {
-        const int g = wave * kDmaLoadsPerWave + i;
-        const bool is_b = g >= kDmaBM / 8;
-        const int row = (is_b ? g - kDmaBM / 8 : g) * 8 + l_row;  // row within the tile
-        const int lc = l_pc ^ ((row >> 1) & 7);                   // logical chunk this lane fetches
+    for (int i = 0; i < kLoadsMax; i++) {
+        const int g = min(i * kWaves + wave, kGroups - 1);
+        const int row2 = g * kRowsPerLoad + l_row;       // 0 .. kBM + kBN - 1 over A then B
+        const bool is_b = row2 >= kBM;
+        const int row = is_b ? row2 - kBM : row2;
+        const int lc = l_pc ^ ((row / kSwzDiv) % kCpr);  // logical chunk this lane fetches
         // rows past the matrix edge are clamped to a valid row; what they produce is never stored
         const int grow = is_b ? min(bn0 + row, N - 1) : min(bm0 + row, M - 1);
         gsrc[i] = (is_b ? B + (size_t)grow * p.ldb : A + (size_t)grow * p.lda) + lc * 8;
     }
-    // The loads are written as inline assembly on purpose: through the builtin the compiler tracks them as LDS
-    // writes and puts s_waitcnt vmcnt(0) in front of every LDS read, which would wait for the prefetched K-tiles as
-    // well; here the waits are placed by hand (vmcnt is decremented in issue order).
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_raw;
-    const unsigned wave_u = __builtin_amdgcn_readfirstlane(wave);
     auto issue = [&](int kt) {
-        const int k0 = min(kt, n_kt - 1) * kDmaBK; // past the end: reload the last tile (keeps the in-flight count constant)
-        const unsigned stage = lds_base + (unsigned)(kt % kDmaStages) * kDmaStageBytes + wave_u * (kDmaLoadsPerWave * 1024);
+        const int k0 = min(kt, n_kt - 1) * kBK; // past the end: reload the last tile (keeps the in-flight count constant)
+        const unsigned dst = lds_base + (unsigned)(kt % kStages) * kStageBytes + (unsigned)wave * 1024;
 #pragma unroll
-        for (int i = 0; i < kDmaLoadsPerWave; i++) {
-            const half_t *src = gsrc[i] + k0;
-            const unsigned dst = stage + i * 1024; // wave-uniform LDS byte address; lane l lands at dst + 16 l
-            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory");
-        }
+        for (int i = 0; i < kLoadsMax; i++)
+            if (i < kLoadsMin || !short_wave) dma16(gsrc[i] + k0, dst + i * (kWaves * 1024));
     };
 
-    float16_t acc[2][2];
+    float16_t acc[2][kNT];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < kNT; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     // operand fragments: lane l supplies row (l % 32), logical chunk 2 * ks + l / 32 of a 32 x 16 slab
     const int frow = lane & 31, fch = lane >> 5;
-    int a_off[2], b_off[2], a_sw[2], b_sw[2];
+    int a_off[2], a_sw[2], b_off[kNT], b_sw[kNT];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        const int ra = wm * 64 + i * 32 + frow, rb = wn * 64 + i * 32 + frow;
-        a_off[i] = ra * 128;
-        a_sw[i] = (ra >> 1) & 7;
-        b_off[i] = kDmaBM * 128 + rb * 128;
-        b_sw[i] = (rb >> 1) & 7;
+        const int ra = wm * 64 + i * 32 + frow;
+        a_off[i] = ra * kRowBytes;
+        a_sw[i] = (ra / kSwzDiv) % kCpr;
+    }
+#pragma unroll
+    for (int j = 0; j < kNT; j++) {
+        const int rb = wn * (32 * kNT) + j * 32 + frow;
+        b_off[j] = (kBM + rb) * kRowBytes;
+        b_sw[j] = (rb / kSwzDiv) % kCpr;
     }
 
-    issue(0);
-    issue(1);
+    // Software pipeline.  LDS: all kStages stages are in flight at the start; at the end of K-tile t the wavefront
+    // waits for K-tile t + 1, passes the barrier (now nobody reads stage t % kStages any more) and refills that stage
+    // with K-tile t + kStages.  Registers: the operand fragments of K-step s + 1 are read from LDS while the MFMAs
+    // of K-step s run (two fragment sets, selected by the parity of the unrolled K-step); the tile change sits in
+    // the middle of the last K-step's MFMAs so that the barrier and the LDS latency behind it stay covered.
+    constexpr int kKS = kBK / 16;
+    static_assert(kKS % 2 == 0, "fragment sets alternate by K-step parity");
+    half8_t af[2][2], bf[2][kNT];
+    auto read_frags = [&](int set, const unsigned char *stage, int ks) {
+        const int lc = ks * 2 + fch;
+#pragma unroll
+        for (int i = 0; i < 2; i++) af[set][i] = *reinterpret_cast<const half8_t *>(stage + a_off[i] + ((lc ^ a_sw[i]) << 4));
+#pragma unroll
+        for (int j = 0; j < kNT; j++) bf[set][j] = *reinterpret_cast<const half8_t *>(stage + b_off[j] + ((lc ^ b_sw[j]) << 4));
+    };
+#pragma unroll
+    for (int t = 0; t < kStages; t++) issue(t);
+    if (short_wave) wait_vmcnt<(kStages - 1) * kLoadsMin>();
+    else wait_vmcnt<(kStages - 1) * kLoadsMax>();
+    __syncthreads();
+    read_frags(0, lds_raw, 0);
     for (int kt = 0; kt < n_kt; kt++) {
-        issue(kt + 2);
-        // K-tile kt was issued two issue() calls ago: at most 2 * kDmaLoadsPerWave newer loads may still be in flight
-        __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * kDmaLoadsPerWave) & 0xF) | (((2 * kDmaLoadsPerWave) >> 4) << 14));
-        __syncthreads();
-        const unsigned char *stage = lds_raw + (kt % kDmaStages) * kDmaStageBytes;
+        const unsigned char *stage = lds_raw + (kt % kStages) * kStageBytes;
 #pragma unroll
-        for (int ks = 0; ks < kDmaBK / 16; ks++) {
-            half8_t af[2], bf[2];
-            const int lc = ks * 2 + fch;
+        for (int ks = 0; ks < kKS; ks++) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if (ks + 1 < kKS) {
+                read_frags(nxt, stage, ks + 1);
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                af[i] = *reinterpret_cast<const half8_t *>(stage + a_off[i] + ((lc ^ a_sw[i]) << 4));
-                bf[i] = *reinterpret_cast<const half8_t *>(stage + b_off[i] + ((lc ^ b_sw[i]) << 4));
+                for (int j = 0; j < kNT; j++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int j = 0; j < kNT / 2; j++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (short_wave) wait_vmcnt<(kStages - 2) * kLoadsMin>();
+                else wait_vmcnt<(kStages - 2) * kLoadsMax>();
+                __syncthreads(); // K-tile kt + 1 is in LDS for everybody, and nobody reads K-tile kt any more
+                issue(kt + kStages);
+                read_frags(nxt, lds_raw + ((kt + 1) % kStages) * kStageBytes, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = kNT / 2; j < kNT; j++)
+#pragma unroll
+                    for (int i = 0; i < 2; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
             }
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70); // drain the clamped tail loads before the block's LDS is released
+    wait_vmcnt<0>(); // drain the clamped tail loads before the block's LDS is released
 
     // ---- epilogue.  Accumulator register v of a 32 x 32 tile: row 8 * (v / 4) + 4 * (lane / 32) + v % 4, col lane % 32
     const int col_in = lane & 31;
@@ -118,8 +173,8 @@ __global__ __launch_bounds__(kDmaThreads) void gemm_f16_dma_kernel(GemmParams p)
 #pragma unroll
     for (int i = 0; i < 2; i++) {
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int c = bn0 + wn * 64 + j * 32 + col_in;
+        for (int j = 0; j < kNT; j++) {
+            const int c = bn0 + wn * (32 * kNT) + j * 32 + col_in;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int r = bm0 + wm * 64 + i * 32 + (v >> 2) * 8 + row_in + (v & 3);
@@ -140,24 +195,66 @@ __global__ __launch_bounds__(kDmaThreads) void gemm_f16_dma_kernel(GemmParams p)
     }
 }
 
-bool gemm_f16_dma_supported(const GemmParams &p) { return p.k >= kDmaBK && (p.k % kDmaBK) == 0 && (p.lda % 8) == 0 && (p.ldb % 8) == 0; }
+bool gemm_f16_dma_supported(const GemmParams &p) { return p.k >= kDmaMinBK && (p.k % kDmaMinBK) == 0 && (p.lda % 8) == 0 && (p.ldb % 8) == 0; }
+
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages>
+static hipError_t launch_dma(const GemmParams &p, hipStream_t s) {
+    constexpr int bm = 64 * kWavesM, bn = 64 * kNT;
+    constexpr size_t lds = (size_t)kStages * (bm + bn) * kBK * 2;
+    static_assert(lds <= 160 * 1024, "LDS of one compute unit");
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr != hipSuccess) return attr;
+    dim3 grid((p.n + bn - 1) / bn, (p.m + bm - 1) / bm, p.batch);
+    hipLaunchKernelGGL((gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages>), grid, dim3(128 * kWavesM), lds, s, p);
+    return hipGetLastError();
+}
+
+template <int kEpi>
+static hipError_t launch_dma_epi(const GemmParams &p, int tile, hipStream_t s) {
+    switch (tile) {
+    case 0: return launch_dma<kEpi, 2, 2, 64, 2>(p, s);  // 128 x 128
+    case 1: return launch_dma<kEpi, 4, 2, 32, 4>(p, s);  // 256 x 128
+    case 2: return launch_dma<kEpi, 4, 3, 32, 4>(p, s);  // 256 x 192
+    case 3: return launch_dma<kEpi, 4, 4, 32, 4>(p, s);  // 256 x 256
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// Tile choice: time ~ (rounds of workgroups over the compute units) x (work per workgroup) / (efficiency of the tile);
+// larger tiles are more efficient (less L2 -> LDS traffic per flop) but leave compute units idle on small outputs.
+static int choose_tile(const GemmParams &p) {
+    static const int forced = getenv("RLLAMA_HIP_GEMM_TILE") ? atoi(getenv("RLLAMA_HIP_GEMM_TILE")) : -1;
+    if (forced >= 1 && forced <= 3) return forced;
+    if (forced == 0 && p.k % 64 == 0) return 0;
+    static const int n_cu = [] {
+        int dev = 0, cu = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev);
+        return cu > 0 ? cu : 256;
+    }();
+    const int bms[4] = {128, 256, 256, 256}, bns[4] = {128, 128, 192, 256};
+    const double eff[4] = {1.0, 0.92, 1.23, 1.15}; // relative throughput of a busy compute unit, measured on 7B shapes
+    int best = -1;
+    double best_t = 0.0;
+    for (int t = 0; t < 4; t++) {
+        if (t == 0 && p.k % 64 != 0) continue;
+        const long blocks = (long)((p.n + bns[t] - 1) / bns[t]) * ((p.m + bms[t] - 1) / bms[t]) * p.batch;
+        const long rounds = (blocks + n_cu - 1) / n_cu;
+        const double time = (double)rounds * bms[t] * bns[t] / eff[t];
+        if (best < 0 || time < best_t) { best = t; best_t = time; }
+    }
+    return best;
+}
 
 hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s) {
     if (!gemm_f16_dma_supported(p) || p.m <= 0 || p.n <= 0 || p.batch < 1) return hipErrorInvalidValue;
-    const size_t lds = (size_t)kDmaStages * kDmaStageBytes;
-    dim3 grid((p.n + kDmaBN - 1) / kDmaBN, (p.m + kDmaBM - 1) / kDmaBM, p.batch);
-    auto go = [&](auto kern) -> hipError_t {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, grid, dim3(kDmaThreads), lds, s, p);
-        return hipGetLastError();
-    };
+    const int tile = choose_tile(p);
     switch (epilogue) {
-    case kGemmEpiF16: return go(gemm_f16_dma_kernel<kGemmEpiF16>);
-    case kGemmEpiF32: return go(gemm_f16_dma_kernel<kGemmEpiF32>);
+    case kGemmEpiF16: return launch_dma_epi<kGemmEpiF16>(p, tile, s);
+    case kGemmEpiF32: return launch_dma_epi<kGemmEpiF32>(p, tile, s);
     case kGemmEpiResAddF32:
         if (p.residual == nullptr || p.batch != 1) return hipErrorInvalidValue;
-        return go(gemm_f16_dma_kernel<kGemmEpiResAddF32>);
+        return launch_dma_epi<kGemmEpiResAddF32>(p, tile, s);
     default: return hipErrorInvalidValue;
     }
 }

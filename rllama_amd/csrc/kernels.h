@@ -91,7 +91,7 @@ struct GemmParams {
 };
 
 hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s);
-// fast path (gemm_dma.hip): k % 64 == 0; launch_gemm_f16 picks it when it applies
+// fast path (gemm_dma.hip): k % 32 == 0; launch_gemm_f16 picks it when it applies
 bool gemm_f16_dma_supported(const GemmParams &p);
 hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s);
 
