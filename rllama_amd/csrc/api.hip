@@ -78,11 +78,12 @@ struct Layer {
 struct PrefillScratch {
     int n_cap = 0;       // rows the buffers are sized for
     int t_pad = 0;       // n_cap rounded up to 64: row stride of scores / probabilities / transposed V
-    float *x = nullptr, *h = nullptr, *scores = nullptr, *o = nullptr;
-    void *xn = nullptr, *qkv = nullptr, *q_hi = nullptr, *q_lo = nullptr, *v_t = nullptr, *p_hi = nullptr, *p_lo = nullptr, *a = nullptr;
+    float *x = nullptr, *h = nullptr, *scores = nullptr;
+    // q2: rows [q hi | q lo] of 2 head_dim halves; p2: rows [P hi | P lo] of 2 t_pad halves (one GEMM sums both parts)
+    void *xn = nullptr, *qkv = nullptr, *q2 = nullptr, *v_t = nullptr, *p2 = nullptr, *a = nullptr;
     void *g = nullptr, *u = nullptr, *mm = nullptr;
     void release() {
-        void *all[] = {x, h, scores, o, xn, qkv, q_hi, q_lo, v_t, p_hi, p_lo, a, g, u, mm};
+        void *all[] = {x, h, scores, xn, qkv, q2, v_t, p2, a, g, u, mm};
         for (void *b : all)
             if (b) (void)hipFree(b);
         *this = PrefillScratch();
@@ -794,13 +795,10 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     A((void **)&S.h, N * d * 4);
     A((void **)&S.xn, N * d * 2);
     A((void **)&S.qkv, N * 3 * d * 2);
-    A((void **)&S.q_hi, N * d * 2);
-    A((void **)&S.q_lo, N * d * 2);
+    A((void **)&S.q2, N * d * 2 * 2);
     A((void **)&S.v_t, H * hd * tp * 2);
     A((void **)&S.scores, H * N * tp * 4);
-    A((void **)&S.p_hi, H * N * tp * 2);
-    A((void **)&S.p_lo, H * N * tp * 2);
-    A((void **)&S.o, N * d * 4);
+    A((void **)&S.p2, H * N * tp * 2 * 2);
     A((void **)&S.a, N * d * 2);
     A((void **)&S.g, N * F * 2);
     A((void **)&S.u, N * F * 2);
@@ -856,8 +854,9 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         PrefillRopeParams rp{};
         rp.qkv = S.qkv;
         rp.freqs = m->freqs;
-        rp.q_hi = S.q_hi;
-        rp.q_lo = S.q_lo;
+        rp.q_hi = S.q2;
+        rp.q_lo = (char *)S.q2 + (size_t)hd * 2;
+        rp.q_stride = 2 * hd;
         rp.cache_k = ck;
         rp.cache_v = cv;
         rp.cache_f16 = 1;
@@ -868,46 +867,50 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         rp.max_seq_len = P.max_seq_len;
         rp.t_pad = tp;
         HIP_TRY(launch_rope_kv_prefill(rp, st));
-        // scores[h] = q[h] . K[h]^T, accumulated over the hi and lo parts of q
-        for (int part = 0; part < 2; part++) {
+        // scores[h] = q[h] . K[h]^T summed over the hi and lo parts of q: one pass that skips the tiles above the
+        // diagonal where the fast GEMM takes head_dim as a K segment, else one accumulating pass per part
+        const bool one_pass = hd % 64 == 0;
+        for (int part = 0; part < (one_pass ? 1 : 2); part++) {
             GemmParams g{};
-            g.a = (const _Float16 *)(part == 0 ? S.q_hi : S.q_lo);
+            g.a = (const _Float16 *)S.q2 + (size_t)part * hd;
             g.b = (const _Float16 *)ck;
             g.c = S.scores;
             g.m = n;
             g.n = n;
-            g.k = hd;
-            g.lda = hd;
+            g.k = one_pass ? 2 * hd : hd;
+            g.k_seg = one_pass ? hd : 0;
+            g.causal = one_pass ? 1 : 0;
+            g.accumulate = part;
+            g.lda = 2 * hd;
             g.ldb = hd;
             g.ldc = tp;
             g.batch = H;
-            g.stride_a = (size_t)n * hd;
+            g.stride_a = (size_t)n * 2 * hd;
             g.stride_b = (size_t)P.max_seq_len * hd;
             g.stride_c = (size_t)n * tp;
-            g.accumulate = part;
             HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
         }
-        HIP_TRY(launch_causal_softmax(S.scores, S.p_hi, S.p_lo, H, n, tp, hd, st));
-        // out[h] = P[h] . V[h], accumulated over the hi and lo parts of P
-        for (int part = 0; part < 2; part++) {
+        HIP_TRY(launch_causal_softmax(S.scores, S.p2, (char *)S.p2 + (size_t)tp * 2, H, n, tp, 2 * tp, hd, st));
+        {   // out[h] = P[h] . V[h] summed over the hi and lo parts of P, rounded to f16 and written as columns
+            // h * hd .. of the [n x dim] input of wo (the concat of heads and the rounding point of transformer.rs:783-796)
             GemmParams g{};
-            g.a = (const _Float16 *)(part == 0 ? S.p_hi : S.p_lo);
+            g.a = (const _Float16 *)S.p2;
             g.b = (const _Float16 *)S.v_t;
-            g.c = S.o;
+            g.c = S.a;
             g.m = n;
             g.n = hd;
-            g.k = tp;
-            g.lda = tp;
+            g.k = 2 * tp;
+            g.k_seg = tp;
+            g.causal = 2;
+            g.lda = 2 * tp;
             g.ldb = tp;
-            g.ldc = hd;
+            g.ldc = d;
             g.batch = H;
-            g.stride_a = (size_t)n * tp;
+            g.stride_a = (size_t)n * 2 * tp;
             g.stride_b = (size_t)hd * tp;
-            g.stride_c = (size_t)n * hd;
-            g.accumulate = part;
-            HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
+            g.stride_c = (size_t)hd;
+            HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
         }
-        HIP_TRY(launch_attn_out_f16(S.o, S.a, n, H, hd, st));
         if ((rc = gemm(S.a, d, L.wo.p, d, S.h, d, n, d, d, kGemmEpiResAddF32, S.x)) != RLH_OK) return rc;     // h = x + wo(att)
         HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.h, (const float *)L.ffn_norm.p, n, d, eps, st));
         if ((rc = gemm(S.xn, d, L.w1.p, d, S.g, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;

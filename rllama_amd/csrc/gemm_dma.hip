@@ -63,13 +63,19 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     const half_t *A = p.a + zb * p.stride_a;
     const half_t *B = p.b + zb * p.stride_b;
     const int M = p.m, N = p.n, K = p.k;
-    const int n_kt = K / kBK;
+    if (p.causal == 1 && bn0 > bm0 + kBM - 1) return; // the whole tile lies above the diagonal (uniform for the workgroup)
+    // K-tiles: n_seg segments of tps tiles each; A's k runs on from segment to segment, B's starts over
+    const int seg_len = p.k_seg > 0 ? p.k_seg : K;
+    const int seg_used = p.causal == 2 ? min(seg_len, (bm0 + kBM + kBK - 1) / kBK * kBK) : seg_len;
+    const int tps = seg_used / kBK;
+    const int n_kt = (K / seg_len) * tps;
 
     // ---- staging: a stage holds rows 0 .. kBM-1 of A then rows 0 .. kBN-1 of B, kRowBytes each.  Load i of
     //      wavefront w moves row group i * kWaves + w; lane l of a group: row l / kCpr, physical chunk l % kCpr.
     const int l_row = lane / kCpr, l_pc = lane % kCpr;
     const bool short_wave = kLoadsMax != kLoadsMin && (kLoadsMax - 1) * kWaves + wave >= kGroups; // one load fewer
     const half_t *gsrc[kLoadsMax];
+    bool src_is_b[kLoadsMax];
 #pragma unroll
     for (int i = 0; i < kLoadsMax; i++) {
         const int g = min(i * kWaves + wave, kGroups - 1);
@@ -80,14 +86,25 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         // rows past the matrix edge are clamped to a valid row; what they produce is never stored
         const int grow = is_b ? min(bn0 + row, N - 1) : min(bm0 + row, M - 1);
         gsrc[i] = (is_b ? B + (size_t)grow * p.ldb : A + (size_t)grow * p.lda) + lc * 8;
+        src_is_b[i] = is_b;
     }
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_raw;
-    auto issue = [&](int kt) {
-        const int k0 = min(kt, n_kt - 1) * kBK; // past the end: reload the last tile (keeps the in-flight count constant)
+    int iss_t = 0, iss_ka = 0, iss_kb = 0; // the K-tile the next issue() loads: index within its segment, k offsets in A and B
+    auto issue = [&](int kt) {             // called for kt = 0, 1, 2, ... in this order
         const unsigned dst = lds_base + (unsigned)(kt % kStages) * kStageBytes + (unsigned)wave * 1024;
 #pragma unroll
         for (int i = 0; i < kLoadsMax; i++)
-            if (i < kLoadsMin || !short_wave) dma16(gsrc[i] + k0, dst + i * (kWaves * 1024));
+            if (i < kLoadsMin || !short_wave) dma16(gsrc[i] + (src_is_b[i] ? iss_kb : iss_ka), dst + i * (kWaves * 1024));
+        if (kt + 1 < n_kt) { // past the end the last tile is loaded again (keeps the in-flight count constant)
+            if (++iss_t == tps) {
+                iss_t = 0;
+                iss_ka += seg_len - (tps - 1) * kBK;
+                iss_kb = 0;
+            } else {
+                iss_ka += kBK;
+                iss_kb += kBK;
+            }
+        }
     };
 
     float16_t acc[2][kNT];
@@ -170,24 +187,40 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // ---- epilogue.  Accumulator register v of a 32 x 32 tile: row 8 * (v / 4) + 4 * (lane / 32) + v % 4, col lane % 32
     const int col_in = lane & 31;
     const int row_in = (lane >> 5) * 4;
+    auto out_row = [&](int i, int v) { return bm0 + wm * 64 + i * 32 + (v >> 2) * 8 + row_in + (v & 3); };
+    auto out_col = [&](int j) { return bn0 + wn * (32 * kNT) + j * 32 + col_in; };
+    // What the epilogue adds to (the residual, or C itself when accumulating) is loaded in batches of one column
+    // tile: C may alias the residual, so a load issued between the stores would wait for the store before it.
+    [[maybe_unused]] const float *prev_src = nullptr;
+    if constexpr (kEpi == kGemmEpiResAddF32) prev_src = p.residual;
+    if constexpr (kEpi == kGemmEpiF32) prev_src = p.accumulate ? reinterpret_cast<const float *>(p.c) + zb * p.stride_c : nullptr;
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (int j = 0; j < kNT; j++) {
+        const int c = out_col(j);
+        [[maybe_unused]] float16_t prev[2];
+        if constexpr (kEpi != kGemmEpiF16) {
 #pragma unroll
-        for (int j = 0; j < kNT; j++) {
-            const int c = bn0 + wn * (32 * kNT) + j * 32 + col_in;
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = out_row(i, v);
+                    prev[i][v] = (prev_src != nullptr && r < M && c < N) ? prev_src[(size_t)r * p.ldc + c] : 0.0f;
+                }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int r = bm0 + wm * 64 + i * 32 + (v >> 2) * 8 + row_in + (v & 3);
+                const int r = out_row(i, v);
                 if (r < M && c < N) {
                     const float val = acc[i][j][v];
                     const size_t off = zb * p.stride_c + (size_t)r * p.ldc + c;
                     if constexpr (kEpi == kGemmEpiF16) {
                         reinterpret_cast<half_t *>(p.c)[off] = (half_t)val; // tensor.rs:1623-1643
                     } else if constexpr (kEpi == kGemmEpiF32) {
-                        float *cp = reinterpret_cast<float *>(p.c) + off;
-                        *cp = p.accumulate ? (*cp + val) : val;
+                        reinterpret_cast<float *>(p.c)[off] = prev[i][v] + val;
                     } else { // kGemmEpiResAddF32: residual add of transformer.rs:442 / :445 on the f16-rounded product
-                        reinterpret_cast<float *>(p.c)[off] = p.residual[(size_t)r * p.ldc + c] + f16r(val);
+                        reinterpret_cast<float *>(p.c)[off] = prev[i][v] + f16r(val);
                     }
                 }
             }
@@ -195,7 +228,11 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     }
 }
 
-bool gemm_f16_dma_supported(const GemmParams &p) { return p.k >= kDmaMinBK && (p.k % kDmaMinBK) == 0 && (p.lda % 8) == 0 && (p.ldb % 8) == 0; }
+bool gemm_f16_dma_supported(const GemmParams &p) {
+    if (p.k < kDmaMinBK || (p.k % kDmaMinBK) != 0 || (p.lda % 8) != 0 || (p.ldb % 8) != 0) return false;
+    if (p.k_seg < 0 || (p.k_seg > 0 && ((p.k % p.k_seg) != 0 || (p.k_seg % 64) != 0))) return false;
+    return p.causal >= 0 && p.causal <= 2;
+}
 
 template <int kEpi, int kWavesM, int kNT, int kBK, int kStages>
 static hipError_t launch_dma(const GemmParams &p, hipStream_t s) {

@@ -88,6 +88,12 @@ struct GemmParams {
     int batch;              // grid.z; element strides between batch items:
     size_t stride_a, stride_b, stride_c;
     int accumulate;         // kGemmEpiF32 only
+    // fast path only (gemm_dma.hip); 0 = off:
+    int k_seg;              // K is made of K / k_seg segments: A's k index runs through all of them, B's wraps (k % k_seg).
+                            // Sums sum_s A_s * B^T in one pass (A = [hi | lo] halves of an fp32 operand against one B).
+    int causal;             // 1: C tiles that lie entirely above the diagonal (col > row) are skipped, not written
+                            // 2: of every segment only k < (last row of the C tile) + 1, rounded up to the K-tile, is used
+                            //    (A holds zeros beyond the diagonal: causal probabilities times V)
 };
 
 hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s);
@@ -99,17 +105,18 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s)
 struct PrefillRopeParams {
     const void *qkv;        // [n x 3 dim] f16
     const float2 *freqs;    // [max_seq_len x head_dim/2]
-    void *q_hi, *q_lo;      // [n_heads][n][head_dim] f16
+    void *q_hi, *q_lo;      // [n_heads][n] rows of head_dim f16, q_stride halves apart
     void *cache_k, *cache_v; // this layer: [n_heads][max_seq_len][head_dim]
     int cache_f16;
     void *v_t;              // [n_heads][head_dim][t_pad] f16
     int n, dim, head_dim, max_seq_len, t_pad;
+    int q_stride;
 };
 hipError_t launch_embed_rows(const void *table, int table_f16, const int32_t *tokens_dev, int n, int dim, float *x, hipStream_t s);
 hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s);
 hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s);
-hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int head_dim, hipStream_t s);
-hipError_t launch_attn_out_f16(const float *o, void *a, int n, int n_heads, int head_dim, hipStream_t s);
+// scores rows are t_pad floats apart, the probability rows (hi and lo alike) p_stride halves
+hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int p_stride, int head_dim, hipStream_t s);
 hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s);
 
 hipError_t launch_embed(const void *table, int table_f16, int dim, const DecodeState *state, float *x, hipStream_t s);

@@ -44,7 +44,7 @@ hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int 
 }
 
 // qkv [n x 3 dim] f16 (rows = tokens at positions 0..n-1) ->
-//   q after RoPE, split hi/lo, head-major [head][n][head_dim]
+//   q after RoPE, split hi/lo, head-major [head][n] rows of head_dim, q_stride halves apart
 //   K (after RoPE) and V into the cache [head][max_seq_len][head_dim] at positions 0..n-1
 //   V transposed [head][head_dim][t_pad] (positions contiguous) as the B operand of P.V
 __global__ void rope_kv_prefill_kernel(PrefillRopeParams p) {
@@ -63,7 +63,7 @@ __global__ void rope_kv_prefill_kernel(PrefillRopeParams p) {
         // q
         float a, b;
         rope_pair((float)row[j], (float)row[j + 1], f, a, b);
-        const size_t qo = ((size_t)head * p.n + r) * p.head_dim + 2 * c;
+        const size_t qo = ((size_t)head * p.n + r) * p.q_stride + 2 * c;
         half_t *qhi = reinterpret_cast<half_t *>(p.q_hi), *qlo = reinterpret_cast<half_t *>(p.q_lo);
         const half_t ah = (half_t)a, bh = (half_t)b;
         qhi[qo] = ah;
@@ -100,59 +100,64 @@ hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s) {
     return hipGetLastError();
 }
 
-// Scores [head][n][t_pad] f32 (raw q.k) -> causal softmax probabilities split hi/lo f16 [head][n][t_pad].
+// Scores [head][n][t_pad] f32 (raw q.k) -> causal softmax probabilities split hi/lo f16, rows p_stride halves apart.
 // scalar_multiply_f32(1/sqrt(hd)), + full_triu mask, softmax (transformer.rs:768-779; tensor.rs:496-508, 479-494);
 // evaluated with the row maximum subtracted, which is the same function wherever the reference's is finite.
-// One wavefront per row; masked and padded columns get probability 0.
+// One wavefront per row.  Masked columns get probability 0 up to the next multiple of 256 columns (what a
+// causal P.V product with row tiles of at most 256 reads); columns past that are left as they are.
+constexpr int kSoftmaxRegs = 32; // scores a lane keeps in registers: rows up to 64 * 32 columns are read once
 __global__ __launch_bounds__(256) void causal_softmax_kernel(const float *scores, half_t *p_hi, half_t *p_lo, size_t total_rows, int n, int t_pad,
-                                                             float scale) {
+                                                             int p_stride, float scale) {
     const int lane = threadIdx.x & 63;
     const size_t row_id = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6); // over heads * n
     if (row_id >= total_rows) return;                                  // whole wavefronts leave together
     const int r = (int)(row_id % (size_t)n);                           // row r attends to columns 0..r
     const float *srow = scores + row_id * t_pad;
-    half_t *hi = p_hi + row_id * t_pad;
-    half_t *lo = p_lo + row_id * t_pad;
+    half_t *hi = p_hi + row_id * p_stride;
+    half_t *lo = p_lo + row_id * p_stride;
+    const int c_end = min(t_pad, (r + 256) & ~255);
+    auto put = [&](int c, float pv) {
+        const half_t h = (half_t)pv;
+        hi[c] = h;
+        lo[c] = (half_t)(pv - (float)h);
+    };
+    if (r < 64 * kSoftmaxRegs) {
+        float v[kSoftmaxRegs];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < kSoftmaxRegs; i++) {
+            const int c = lane + 64 * i;
+            v[i] = c <= r ? srow[c] * scale : -INFINITY;
+            mx = fmaxf(mx, v[i]);
+        }
+        mx = wave_max(mx);
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kSoftmaxRegs; i++) {
+            v[i] = expf(v[i] - mx); // masked columns: exp(-inf) = 0
+            sum += v[i];
+        }
+        sum = wave_sum(sum);
+#pragma unroll
+        for (int i = 0; i < kSoftmaxRegs; i++) {
+            const int c = lane + 64 * i;
+            if (c < c_end) put(c, v[i] / sum);
+        }
+        return;
+    }
     float mx = -INFINITY;
     for (int c = lane; c <= r; c += 64) mx = fmaxf(mx, srow[c] * scale);
     mx = wave_max(mx);
     float sum = 0.0f;
     for (int c = lane; c <= r; c += 64) sum += expf(srow[c] * scale - mx);
     sum = wave_sum(sum);
-    for (int c = lane; c < t_pad; c += 64) {
-        float pv = 0.0f;
-        if (c <= r) pv = expf(srow[c] * scale - mx) / sum;
-        const half_t h = (half_t)pv;
-        hi[c] = h;
-        lo[c] = (half_t)(pv - (float)h);
-    }
+    for (int c = lane; c < c_end; c += 64) put(c, c <= r ? expf(srow[c] * scale - mx) / sum : 0.0f);
 }
 
-hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int head_dim, hipStream_t s) {
+hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int p_stride, int head_dim, hipStream_t s) {
     const size_t rows = (size_t)n_heads * n;
     hipLaunchKernelGGL(causal_softmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, scores, (half_t *)p_hi, (half_t *)p_lo, rows, n, t_pad,
-                       1.0f / sqrtf((float)head_dim)); // transformer.rs:770
-    return hipGetLastError();
-}
-
-// attention output [head][n][head_dim] f32 -> [n][dim] f16: the concat of heads per row and the f16 rounding
-// point before wo (transformer.rs:783-796)
-__global__ void attn_out_f16_kernel(const float *o, half_t *a, int n, int n_heads, int head_dim) {
-    const size_t total = (size_t)n * n_heads * head_dim;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const int dim = n_heads * head_dim;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int r = (int)(i / dim);
-        const int j = (int)(i - (size_t)r * dim);
-        const int head = j / head_dim, jj = j - head * head_dim;
-        a[i] = (half_t)o[((size_t)head * n + r) * head_dim + jj];
-    }
-}
-
-hipError_t launch_attn_out_f16(const float *o, void *a, int n, int n_heads, int head_dim, hipStream_t s) {
-    const size_t total = (size_t)n * n_heads * head_dim;
-    const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
-    hipLaunchKernelGGL(attn_out_f16_kernel, dim3(blocks), dim3(256), 0, s, o, (half_t *)a, n, n_heads, head_dim);
+                       p_stride, 1.0f / sqrtf((float)head_dim)); // transformer.rs:770
     return hipGetLastError();
 }
 

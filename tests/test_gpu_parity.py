@@ -189,6 +189,20 @@ def test_forward_f16_mode(ctx, shape):
     gm.free()
 
 
+def test_prefill_long_prompt_causal_tiles(ctx):
+    """A prompt long enough that the score matrix spans several GEMM tiles per head (tiles above the diagonal are
+    skipped, the probability product stops at the diagonal) on the large-tile path; compared with the oracle."""
+    shape = Shape(dim=1024, n_layers=1, n_heads=16, ffn_hidden=256, vocab_size=64, max_seq_len=1024)
+    W = synth_weights(shape, seed=43, std=0.05, norm_ones=False)
+    toks = np.random.default_rng(44).integers(0, shape.vocab_size, 1024)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    for n in (1024, 700):
+        want = om.forward(toks[:n], 0, om.make_caches())
+        got = gm.forward(toks[:n], 0, gm.make_caches())
+        assert max_rel_err(got, want) < TOL_F16, (n, max_rel_err(got, want))
+    gm.free()
+
+
 @pytest.mark.parametrize("shape", [TINY, SMALL], ids=["tiny", "small"])
 def test_forward_f32_mode(ctx, shape):
     W = random_f32_weights(shape, seed=23, std=0.08)
@@ -329,7 +343,9 @@ def test_percentage_to_gpu_rule(ctx):
         m.free()
 
 
-@pytest.mark.parametrize("n,m_rows,k", [(2, 3, 8), (33, 65, 72), (128, 128, 64), (130, 200, 192), (16, 2816, 1024), (257, 384, 4096), (1024, 256, 11008)])
+# the last four are sized so that the tile choice lands on the 256 x 192, 256 x 256 and 256 x 128 tiles (with ragged edges)
+@pytest.mark.parametrize("n,m_rows,k", [(2, 3, 8), (33, 65, 72), (128, 128, 64), (130, 200, 192), (16, 2816, 1024), (257, 384, 4096), (1024, 256, 11008),
+                                        (1024, 12288, 64), (1000, 12290, 160), (1024, 16384, 96), (512, 16384, 96)])
 def test_mfma_gemm_f16(ctx, n, m_rows, k):
     """src [n x k] . other[m x k]^T with n > 1 runs on the matrix cores; every element against the oracle's
     f16-rounded dot8 (tensor.rs:1476-1666), including tiles that straddle the matrix edges."""
