@@ -3,17 +3,67 @@
 // the reference prints it (first token apart, then the mean over the rest; src/rllama_main.rs:908-917).
 //
 //   rllama_generate [dim n_layers n_heads ffn_hidden vocab n_prompt n_new [seed]]
+//   rllama_generate --model-path DIR [n_prompt n_new [seed]]     weights from a LLaMA-format directory (--model-path of
+//                                                                 src/rllama_main.rs:44-45); prompt ids are synthetic
+//   rllama_generate --inspect DIR                                 no device needed: parses params.json and every data.pkl
+//                                                                 and prints each tensor's name, shape and a checksum
 //
 // It exists to show (and to compile-check in every build) that the header-only host layer needs nothing but
 // the C ABI.  Exits non-zero with the library's message if there is no gfx950 device.
+#include "model_files.hpp"
 #include "rllama_hip.hpp"
 
 #include <cstdio>
 #include <cstdlib>
 
+static int inspect(const char *dir) {
+    using namespace rllama;
+    const DataSource src = DataSource::from_inferred_source(dir);
+    const ModelParams mp = src.params();
+    printf("params dim=%zu n_heads=%zu n_layers=%zu norm_eps=%g vocab_size=%lld shards=%zu\n", mp.dim, mp.n_heads, mp.n_layers, mp.norm_eps,
+           (long long)mp.vocab_size, src.unpickled().size());
+    if (src.unpickled().empty()) return 0;
+    for (const auto &kv : src.unpickled()[0]->entries) {
+        const std::string &name = kv.first;
+        // how the reference joins the shards of this tensor (src/transformer.rs:490-503, 595-614; src/embedding.rs:37)
+        const bool cols = name.find(".wo.") != std::string::npos || name.find(".w2.") != std::string::npos || name == "tok_embeddings.weight";
+        const bool first = name.find("norm") != std::string::npos;
+        const HalfMatrix m = load_from_pieces(src, name, cols ? FromPiecesDirection::Cols : FromPiecesDirection::Rows, first);
+        uint64_t h = 1469598103934665603ull; // FNV-1a over the little-endian bytes
+        for (uint16_t b : m.bits) {
+            h = (h ^ (b & 0xff)) * 1099511628211ull;
+            h = (h ^ (b >> 8)) * 1099511628211ull;
+        }
+        printf("tensor %s %lld %lld %016llx\n", name.c_str(), (long long)m.rows, (long long)m.cols, (unsigned long long)h);
+    }
+    return 0;
+}
+
 int main(int argc, char **argv) {
+    if (argc >= 3 && std::string(argv[1]) == "--inspect") {
+        try {
+            return inspect(argv[2]);
+        } catch (const std::exception &e) {
+            fprintf(stderr, "rllama_generate: %s\n", e.what());
+            return 1;
+        }
+    }
+    const char *model_path = nullptr;
+    if (argc >= 3 && std::string(argv[1]) == "--model-path") {
+        model_path = argv[2];
+        argv += 2;
+        argc -= 2;
+    }
     size_t dim = 1024, n_layers = 8, n_heads = 16, ffn = 2816, vocab = 32000, n_prompt = 16, n_new = 64;
     uint64_t seed = 0;
+    if (model_path) {
+        if (argc >= 3) {
+            n_prompt = strtoul(argv[1], nullptr, 10);
+            n_new = strtoul(argv[2], nullptr, 10);
+        }
+        if (argc >= 4) seed = strtoull(argv[3], nullptr, 10);
+        argc = 0;
+    }
     if (argc >= 8) {
         dim = strtoul(argv[1], nullptr, 10);
         n_layers = strtoul(argv[2], nullptr, 10);
@@ -27,8 +77,16 @@ int main(int argc, char **argv) {
     try {
         auto cl = std::make_shared<rllama::OpenCL>(true, 0);
         rllama::DataSettings ds = rllama::DataSettings(cl).force_f16().percentage_to_gpu(1.0f);
-        rllama::Transformer tr(dim, n_layers, n_heads, ffn, vocab, n_prompt + n_new, 1e-6, ds);
-        tr.fill_synthetic(seed, 0.02);
+        std::unique_ptr<rllama::Transformer> loaded;
+        if (model_path) {
+            rllama::ModelParams mp;
+            loaded = rllama::load_transformer(model_path, n_prompt + n_new, ds, &mp);
+            vocab = (size_t)mp.vocab_size;
+        } else {
+            loaded = std::make_unique<rllama::Transformer>(dim, n_layers, n_heads, ffn, vocab, n_prompt + n_new, 1e-6, ds);
+            loaded->fill_synthetic(seed, 0.02);
+        }
+        rllama::Transformer &tr = *loaded;
         std::vector<rllama::TokenId> prompt(n_prompt);
         rlh_synth_tokens(seed, 0, n_prompt, 3, (int32_t)vocab, prompt.data());
         rllama::TransformerCaches caches = tr.make_caches();
@@ -40,6 +98,9 @@ int main(int argc, char **argv) {
         printf("Time taken per token (excluding first token): %.3fms\n", ms_tok);
     } catch (const rllama::Error &e) {
         fprintf(stderr, "rllama_generate: %s (status %d)\n", e.what(), e.code);
+        return 1;
+    } catch (const std::exception &e) {
+        fprintf(stderr, "rllama_generate: %s\n", e.what());
         return 1;
     }
     return 0;

@@ -385,3 +385,46 @@ def test_prefill_matrix_core_path_against_token_by_token_and_oracle(ctx):
         nxt = int(toks[n % len(toks)])
         assert max_rel_err(gm.forward([nxt], n, ga), gm.forward([nxt], n, gb)) < TOL_F16
     gm.free()
+
+
+def _checkpoint_tensors(shape, W):
+    """The reference's tensor names -> f16 bits, from a weight dict of common.synth_weights (norms rounded to f16)."""
+    names = {rllama_amd.TOK_EMB: "tok_embeddings.weight", rllama_amd.NORM: "norm.weight", rllama_amd.OUTPUT: "output.weight"}
+    per_layer = {rllama_amd.WQ: "attention.wq", rllama_amd.WK: "attention.wk", rllama_amd.WV: "attention.wv", rllama_amd.WO: "attention.wo",
+                 rllama_amd.W1: "feed_forward.w1", rllama_amd.W2: "feed_forward.w2", rllama_amd.W3: "feed_forward.w3",
+                 rllama_amd.ATTN_NORM: "attention_norm", rllama_amd.FFN_NORM: "ffn_norm"}
+    T, W16 = {}, {}
+    for (kind, layer), arr in W.items():
+        bits = arr if arr.dtype == np.uint16 else arr.astype(np.float16).view(np.uint16)
+        W16[(kind, layer)] = bits
+        name = names[kind] if kind in names else f"layers.{layer}.{per_layer[kind]}.weight"
+        T[name] = bits.reshape(-1) if "norm" in name else bits
+    return T, W16
+
+
+@pytest.mark.parametrize("shards", [1, 2])
+def test_model_loaded_from_checkpoint_directory(ctx, tmp_path, shards):
+    """params.json + consolidated.NN (src/data_source.rs:166-210) -> device model: the loader hands over exactly the bits
+    of the files, so logits equal those of a model filled tensor by tensor; the C++ host loader generates the same ids."""
+    import subprocess
+    from rllama_amd import build, checkpoint
+    shape = SMALL
+    T, W16 = _checkpoint_tensors(shape, synth_weights(shape, seed=51, std=0.08, norm_ones=False))
+    path = str(tmp_path / "model")
+    checkpoint.write_checkpoint(path, {"dim": shape.dim, "multiple_of": 32, "n_heads": shape.n_heads, "n_layers": shape.n_layers,
+                                       "norm_eps": shape.norm_eps, "vocab_size": shape.vocab_size}, T, n_shards=shards)
+    ds = rllama_amd.DataSettings(ctx).force_f16()
+    loaded = checkpoint.load_transformer(ctx, path, ds, shape.max_seq_len)
+    direct = make_gpu(ctx, shape, W16, True)
+    n_prompt, n_new = 9, 12
+    prompt = rllama_amd.synth_tokens(0, n_prompt, 3, shape.vocab_size)
+    a = loaded.forward(prompt, 0, loaded.make_caches())
+    b = direct.forward(prompt, 0, direct.make_caches())
+    assert np.array_equal(a, b)
+    want_ids, _, _ = direct.generate_greedy(prompt, n_new, direct.make_caches())
+    loaded.free()
+    direct.free()
+    r = subprocess.run([build.build_host(), "--model-path", path, str(n_prompt), str(n_new), "0"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    line = [ln for ln in r.stdout.splitlines() if ln.startswith("tokens:")][0]
+    assert [int(t) for t in line.split()[1:]] == [int(t) for t in want_ids]
