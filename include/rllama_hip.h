@@ -155,6 +155,33 @@ int  rlh_generate_greedy(rlh_model *model, rlh_caches *caches, const int32_t *pr
  * time of the n_steps steps on the launch stream. */
 int  rlh_decode_greedy(rlh_model *model, rlh_caches *caches, int n_steps, int32_t *out_tokens, float *ms_total);
 
+/* TokenSampler (src/token_sampler.rs:6-11).  rlh_sampler_default fills in TokenSampler::new()'s values
+ * (:20-29: temperature 0.2, top_p 1.0, top_k 1, repetition_penalty 0.8). */
+typedef struct rlh_sampler_params {
+    float temperature;          /* logits are multiplied by 1 / temperature when it is > 0 (:99-102) */
+    float top_p;
+    int32_t top_k;
+    float repetition_penalty;   /* 1.0 = none */
+} rlh_sampler_params;
+void rlh_sampler_default(rlh_sampler_params *p);
+
+/* TokenSampler::sample up to the random draw (src/token_sampler.rs:83-159), host arithmetic on host logits (needs no
+ * device): the candidates that survive the top-k and top-p cuts, in the order the draw walks them, with their softmax
+ * probabilities; *total_p is their mass.  The reference's loops over "rows" of the transposed logits touch only token 0
+ * (:105, :113, :121): only token 0 is penalised, and its logit ends up as 0; nothing else has a maximum subtracted.
+ * Equal probabilities are ordered by ascending id.  out_ids / out_probs hold `cap` entries; more candidates than
+ * that is RLH_ERR_INVALID.  existing_tokens may be NULL when n_existing is 0. */
+int  rlh_sample_candidates(const float *logits, int vocab, const rlh_sampler_params *p, const int32_t *existing_tokens, int n_existing,
+                           int32_t *out_ids, float *out_probs, int cap, int *n_out, float *total_p);
+/* The whole of TokenSampler::sample (:83-174) with the uniform variate passed in: u in [0, 1] stands for
+ * rng.gen_range(0.0..=total_p) / total_p.  *prob (may be NULL) = the chosen probability / total_p. */
+int  rlh_sample(const float *logits, int vocab, const rlh_sampler_params *p, const int32_t *existing_tokens, int n_existing, float u,
+                int32_t *token, float *prob);
+/* forward + sample: the body of the reference's token loop (src/rllama_main.rs:846-860).  With top_k == 1 the choice is
+ * made by the device argmax (no logits leave the device) and *prob is 1. */
+int  rlh_forward_sample(rlh_model *model, rlh_caches *caches, const int32_t *tokens, int n, int start_pos, const rlh_sampler_params *p,
+                        const int32_t *existing_tokens, int n_existing, float u, int32_t *token, float *prob);
+
 /* ------------------------------------------------------------------------------------------------
  * Op level.  Mirrors OpenCLTensor (src/tensor_opencl_support.rs:134-405) so that a host Tensor can
  * offload single ops, and so that each kernel can be checked alone.  Tensors are dense row-major.

@@ -81,6 +81,8 @@ def lib() -> C.CDLL:
         "orc_freqs_cis": (None, [C.c_int, C.c_int, C.c_double, dp]),
         "orc_rope_row": (None, [fp, C.c_int, C.c_int, dp]),
         "orc_sample_greedy": (C.c_int32, [fp, C.c_int, C.c_float, fp, i32p]),
+        "orc_sample_candidates": (C.c_int32, [fp, C.c_int, C.c_float, C.c_float, C.c_int32, C.c_float, i32p, C.c_int32, i32p, fp, fp]),
+        "orc_sample_pick": (C.c_int32, [i32p, fp, C.c_int32, C.c_float, C.c_float, fp]),
         "orc_set_threads": (None, [C.c_int]),
         "orc_get_threads": (C.c_int, []),
         "orc_set_reference_threading": (None, [C.c_int]),
@@ -232,6 +234,28 @@ def sample_greedy(logits, temperature: float = 1.0):
     ties = C.c_int32(0)
     tok = lib().orc_sample_greedy(_fp(l), l.size, temperature, C.byref(prob), C.byref(ties))
     return int(tok), float(prob.value), int(ties.value)
+
+
+def sample_candidates(logits, temperature: float, top_p: float, top_k: int, repetition_penalty: float, existing_tokens=()):
+    """token_sampler.rs:83-159: (ids, probabilities, total_p) of the candidates the draw chooses from, in draw order."""
+    l = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+    ex = np.ascontiguousarray(existing_tokens, dtype=np.int32).reshape(-1)
+    cap = max(1, min(int(top_k), l.size))
+    ids = np.zeros(cap, np.int32)
+    probs = np.zeros(cap, np.float32)
+    tot = C.c_float(0)
+    n = lib().orc_sample_candidates(_fp(l), l.size, temperature, top_p, int(min(top_k, 2**31 - 1)), repetition_penalty,
+                                    ex.ctypes.data_as(C.POINTER(C.c_int32)), ex.size, ids.ctypes.data_as(C.POINTER(C.c_int32)), _fp(probs), C.byref(tot))
+    return ids[:n].copy(), probs[:n].copy(), float(tot.value)
+
+
+def sample_pick(ids, probs, total_p: float, u: float):
+    """token_sampler.rs:160-173 with the uniform variate u in [0, 1] passed in. Returns (token id, probability / total_p)."""
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    probs = np.ascontiguousarray(probs, dtype=np.float32)
+    prob = C.c_float(0)
+    tok = lib().orc_sample_pick(ids.ctypes.data_as(C.POINTER(C.c_int32)), _fp(probs), ids.size, total_p, u, C.byref(prob))
+    return int(tok), float(prob.value)
 
 
 def set_threads(n: int) -> None:

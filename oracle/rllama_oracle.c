@@ -416,6 +416,90 @@ void orc_rope_row(float *x, int n_heads, int head_dim, const double *fc) {
     }
 }
 
+/* TokenSampler::sample up to the random draw (token_sampler.rs:83-158): the candidates left after the top-k and top-p
+ * cuts, in the order the draw walks them, with their softmax probabilities.  Returns the number of candidates (at most
+ * min(top_k, vocab); out_ids / out_probs must hold that many); *total_p is their probability mass (:159-162).
+ * Ties between equal probabilities are ordered by ascending id (the reference's sort_unstable_by leaves them unspecified). */
+typedef struct { int32_t id; float p; } orc_cand;
+static int orc_cand_cmp(const void *a, const void *b) {
+    const orc_cand *x = (const orc_cand *)a, *y = (const orc_cand *)b;
+    /* token_sampler.rs:131-145: descending by probability, NaN last */
+    int xn = isnan(x->p), yn = isnan(y->p);
+    if (xn || yn) {
+        if (xn && yn) return (x->id > y->id) - (x->id < y->id);
+        return xn ? 1 : -1;
+    }
+    if (x->p > y->p) return -1;
+    if (x->p < y->p) return 1;
+    return (x->id > y->id) - (x->id < y->id);
+}
+
+int32_t orc_sample_candidates(const float *logits_in, int vocab, float temperature, float top_p, int32_t top_k, float repetition_penalty,
+                              const int32_t *existing_tokens, int32_t n_existing, int32_t *out_ids, float *out_probs, float *total_p) {
+    float *l = (float *)malloc(sizeof(float) * (size_t)vocab);
+    orc_cand *c = (orc_cand *)malloc(sizeof(orc_cand) * (size_t)vocab);
+    memcpy(l, logits_in, sizeof(float) * (size_t)vocab);
+    if (temperature > 0.0f) { /* :99-102, scalar_multiply_f32(1.0 / temperature) */
+        float inv = 1.0f / temperature;
+        for (int i = 0; i < vocab; i++) l[i] = l[i] * inv;
+    }
+    /* :104-123.  After the transpose the tensor is 1 x vocab and the three loops run over 0..rows() == 0..1: only
+     * token 0 is penalised (by penalty^count), "maxv" is token 0's value, and only token 0 has it subtracted. */
+    if (repetition_penalty != 1.0f) {
+        int count = 0;
+        for (int i = 0; i < n_existing; i++) count += existing_tokens[i] == 0;
+        if (count > 0) l[0] = l[0] * powf(repetition_penalty, (float)count);
+    }
+    {
+        float maxv = -INFINITY;
+        if (l[0] > maxv) maxv = l[0];
+        l[0] = l[0] - maxv;
+    }
+    float sum = 0.0f; /* :124 softmax (tensor.rs:479-494): no maximum subtracted, sequential f32 sum */
+    for (int i = 0; i < vocab; i++) sum += expf(l[i]);
+    for (int i = 0; i < vocab; i++) {
+        c[i].id = i;
+        c[i].p = expf(l[i]) / sum;
+    }
+    qsort(c, (size_t)vocab, sizeof(orc_cand), orc_cand_cmp);
+    int32_t n = top_k < vocab ? top_k : vocab; /* :147 truncate(top_k) */
+    if (n < 0) n = 0;
+    float acc = 0.0f;
+    for (int32_t i = 0; i < n; i++) { /* :148-155 */
+        acc += c[i].p;
+        if (acc >= top_p) {
+            n = i + 1;
+            break;
+        }
+    }
+    float tot = 0.0f;
+    for (int32_t i = 0; i < n; i++) { /* :156-159 */
+        tot += c[i].p;
+        out_ids[i] = c[i].id;
+        out_probs[i] = c[i].p;
+    }
+    *total_p = tot;
+    free(l);
+    free(c);
+    return n;
+}
+
+/* The draw (token_sampler.rs:160-173) with the uniform variate passed in: p = u * total_p stands for
+ * rng.gen_range(0.0..=total_p).  Returns the token id, *prob = its probability / total_p. */
+int32_t orc_sample_pick(const int32_t *ids, const float *probs, int32_t n, float total_p, float u, float *prob) {
+    float p = total_p > 0.0f ? u * total_p : 0.0f;
+    float acc = 0.0f;
+    for (int32_t i = 0; i < n; i++) {
+        acc += probs[i];
+        if (acc >= p) {
+            if (prob) *prob = probs[i] / total_p;
+            return ids[i];
+        }
+    }
+    if (prob) *prob = 0.0f;
+    return 0;
+}
+
 int32_t orc_sample_greedy(const float *logits_in, int vocab, float temperature, float *prob, int32_t *n_ties) {
     float *l = (float *)malloc(sizeof(float) * (size_t)vocab);
     memcpy(l, logits_in, sizeof(float) * (size_t)vocab);

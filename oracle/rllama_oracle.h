@@ -106,6 +106,10 @@ void orc_rope_row(float *x, int n_heads, int head_dim, const double *freqs_cis_a
  * receives how many ids share the top probability (the reference's sort_unstable_by does not
  * define which of them wins; this picks the lowest id). */
 int32_t orc_sample_greedy(const float *logits, int vocab, float temperature, float *prob, int32_t *n_ties);
+/* token_sampler.rs:83-174 in two halves: the candidate list after the top-k / top-p cuts, and the draw with the uniform variate passed in */
+int32_t orc_sample_candidates(const float *logits, int vocab, float temperature, float top_p, int32_t top_k, float repetition_penalty,
+                              const int32_t *existing_tokens, int32_t n_existing, int32_t *out_ids, float *out_probs, float *total_p);
+int32_t orc_sample_pick(const int32_t *ids, const float *probs, int32_t n, float total_p, float u, float *prob);
 
 /* ---- model level ---- */
 

@@ -9,7 +9,7 @@ fallback: every method is one call into the library, and a missing library or de
 from __future__ import annotations
 
 import ctypes as C
-from typing import Optional, Sequence
+from typing import Optional, Sequence, Tuple
 
 import numpy as np
 
@@ -229,6 +229,16 @@ class Transformer:
                                             out.ctypes.data_as(C.POINTER(C.c_int32)), C.byref(a), C.byref(b)))
         return out, a.value, b.value
 
+    def forward_sample(self, tokens: Sequence[int], start_pos: int, caches: TransformerCaches, sampler: "TokenSampler",
+                       existing_tokens: Sequence[int], rng: np.random.Generator):
+        """forward + TokenSampler::sample, the body of the token loop (src/rllama_main.rs:846-860). Returns (id, probability)."""
+        toks = np.ascontiguousarray(tokens, dtype=np.int32)
+        ex = np.ascontiguousarray(existing_tokens, dtype=np.int32).reshape(-1)
+        tok, prob = C.c_int32(0), C.c_float(0)
+        check(self._lib.rlh_forward_sample(self._h, caches._h, toks.ctypes.data_as(C.POINTER(C.c_int32)), toks.size, start_pos, C.byref(sampler._p),
+                                           ex.ctypes.data_as(C.POINTER(C.c_int32)), ex.size, float(rng.random(dtype=np.float32)), C.byref(tok), C.byref(prob)))
+        return int(tok.value), float(prob.value)
+
     def decode_greedy(self, n_steps: int, caches: TransformerCaches):
         """Continues the greedy loop on the device for n_steps tokens. Returns (ids, HIP-event ms for the n_steps)."""
         out = np.empty(n_steps, dtype=np.int32)
@@ -361,6 +371,72 @@ class Tensor:
             self.free()
         except Exception:
             pass
+
+
+class TokenSampler:
+    """TokenSampler (src/token_sampler.rs:6-174): builder-style settings, sampling done by the library's host arithmetic.
+    The uniform variate comes from the caller's generator (the reference draws from rand::thread_rng)."""
+
+    def __init__(self):
+        self._p = _lib.SamplerParams()
+        _lib.load().rlh_sampler_default(C.byref(self._p))  # TokenSampler::new(), :20-29
+
+    def _with(self, **kw) -> "TokenSampler":
+        t = TokenSampler()
+        t._p = _lib.SamplerParams(self._p.temperature, self._p.top_p, self._p.top_k, self._p.repetition_penalty)
+        for k, v in kw.items():
+            setattr(t._p, k, v)
+        return t
+
+    def temperature(self, v: float) -> "TokenSampler":
+        return self._with(temperature=v)
+
+    def top_p(self, v: float) -> "TokenSampler":
+        return self._with(top_p=v)
+
+    def top_k(self, v: int) -> "TokenSampler":
+        return self._with(top_k=int(min(v, 2**31 - 1)))
+
+    def repetition_penalty(self, v: float) -> "TokenSampler":
+        return self._with(repetition_penalty=v)
+
+    def get_temperature(self) -> float:
+        return self._p.temperature
+
+    def get_top_p(self) -> float:
+        return self._p.top_p
+
+    def get_top_k(self) -> int:
+        return self._p.top_k
+
+    def get_repetition_penalty(self) -> float:
+        return self._p.repetition_penalty
+
+    @staticmethod
+    def _existing(existing_tokens):
+        ex = np.ascontiguousarray(existing_tokens, dtype=np.int32).reshape(-1)
+        return ex, ex.ctypes.data_as(C.POINTER(C.c_int32))
+
+    def candidates(self, logits: np.ndarray, existing_tokens: Sequence[int] = ()):
+        """(ids, probabilities, total_p) of what the draw chooses from, in draw order (:83-159)."""
+        l = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+        ex, exp_ = self._existing(existing_tokens)
+        cap = max(1, min(self._p.top_k, l.size))
+        ids, probs = np.zeros(cap, np.int32), np.zeros(cap, np.float32)
+        n, tot = C.c_int(0), C.c_float(0)
+        check(_lib.load().rlh_sample_candidates(l.ctypes.data_as(C.POINTER(C.c_float)), l.size, C.byref(self._p), exp_, ex.size,
+                                                ids.ctypes.data_as(C.POINTER(C.c_int32)), probs.ctypes.data_as(C.POINTER(C.c_float)), cap,
+                                                C.byref(n), C.byref(tot)))
+        return ids[:n.value].copy(), probs[:n.value].copy(), float(tot.value)
+
+    def sample(self, logits: np.ndarray, existing_tokens: Sequence[int], rng: np.random.Generator) -> Tuple[int, float]:
+        """sample(logits, tokenizer, existing_tokens) -> (token id, probability) (:83-174)."""
+        l = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+        ex, exp_ = self._existing(existing_tokens)
+        tok, prob = C.c_int32(0), C.c_float(0)
+        check(_lib.load().rlh_sample(l.ctypes.data_as(C.POINTER(C.c_float)), l.size, C.byref(self._p), exp_, ex.size, float(rng.random(dtype=np.float32)),
+                                     C.byref(tok), C.byref(prob)))
+        return int(tok.value), float(prob.value)
 
 
 # -- synthetic inputs (host side of csrc/synth.h; needs no device) --------------------------------------

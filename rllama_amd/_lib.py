@@ -30,6 +30,10 @@ class ModelParams(C.Structure):
     ]
 
 
+class SamplerParams(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("top_k", C.c_int32), ("repetition_penalty", C.c_float)]
+
+
 _vp = C.c_void_p
 _vpp = C.POINTER(C.c_void_p)
 _i32p = C.POINTER(C.c_int32)
@@ -60,6 +64,10 @@ SIGNATURES = {
     "rlh_forward_greedy": (C.c_int, [_vp, _vp, _i32p, C.c_int, C.c_int, _i32p]),
     "rlh_generate_greedy": (C.c_int, [_vp, _vp, _i32p, C.c_int, C.c_int, _i32p, _fp, _fp]),
     "rlh_decode_greedy": (C.c_int, [_vp, _vp, C.c_int, _i32p, _fp]),
+    "rlh_sampler_default": (None, [C.POINTER(SamplerParams)]),
+    "rlh_sample_candidates": (C.c_int, [_fp, C.c_int, C.POINTER(SamplerParams), _i32p, C.c_int, _i32p, _fp, C.c_int, _ip, _fp]),
+    "rlh_sample": (C.c_int, [_fp, C.c_int, C.POINTER(SamplerParams), _i32p, C.c_int, C.c_float, _i32p, _fp]),
+    "rlh_forward_sample": (C.c_int, [_vp, _vp, _i32p, C.c_int, C.c_int, C.POINTER(SamplerParams), _i32p, C.c_int, C.c_float, _i32p, _fp]),
     "rlh_tensor_upload": (C.c_int, [_vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, _vpp]),
     "rlh_tensor_alloc": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, _vpp]),
     "rlh_tensor_download": (C.c_int, [_vp, _vp, C.c_int, _vpp]),

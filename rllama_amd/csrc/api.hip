@@ -37,6 +37,10 @@ static int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+namespace rlh {
+int set_error(int code, const char *msg) { return fail(code, "%s", msg); } // for the library's other translation units
+} // namespace rlh
+
 #define HIP_TRY(expr)                                                                                     \
     do {                                                                                                  \
         hipError_t _e = (expr);                                                                           \
@@ -992,6 +996,24 @@ extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *to
     m->next_pos = start_pos + n;
     m->greedy_caches = c;
     return RLH_OK;
+}
+
+extern "C" int rlh_forward_sample(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, const rlh_sampler_params *sp,
+                                  const int32_t *existing_tokens, int n_existing, float u, int32_t *token, float *prob) {
+    if (!sp || !token) return fail(RLH_ERR_INVALID, "rlh_forward_sample: NULL argument");
+    if (sp->top_k == 1) {
+        // one candidate: the draw cannot choose.  Which one it is does not depend on temperature (> 0 keeps the order, and
+        // token 0 sits at exactly 0 either way) nor on the penalty (it only reaches token 0, whose value is then shifted to 0),
+        // so the device argmax with the token-0 rule decides (token_sampler.rs:99-147).
+        const int rc = rlh_forward_greedy(m, c, tokens, n, start_pos, token);
+        if (rc == RLH_OK && prob) *prob = 1.0f; // v.1 / total_p with a single candidate (:170)
+        return rc;
+    }
+    if (!m) return fail(RLH_ERR_INVALID, "rlh_forward_sample: NULL argument");
+    std::vector<float> logits((size_t)m->prm.vocab_size);
+    int rc = rlh_forward(m, c, tokens, n, start_pos, logits.data());
+    if (rc != RLH_OK) return rc;
+    return rlh_sample(logits.data(), m->prm.vocab_size, sp, existing_tokens, n_existing, u, token, prob);
 }
 
 extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *prompt, int n_prompt, int n_new, int32_t *out_tokens,

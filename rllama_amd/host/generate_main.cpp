@@ -5,6 +5,8 @@
 //   rllama_generate [dim n_layers n_heads ffn_hidden vocab n_prompt n_new [seed]]
 //   rllama_generate --model-path DIR [n_prompt n_new [seed]]     weights from a LLaMA-format directory (--model-path of
 //                                                                 src/rllama_main.rs:44-45); prompt ids are synthetic
+//   ... --sample TOP_K TEMPERATURE TOP_P REPETITION_PENALTY      (before the other arguments) token loop with
+//                                                                 TokenSampler instead of the device-resident greedy loop
 //   rllama_generate --inspect DIR                                 no device needed: parses params.json and every data.pkl
 //                                                                 and prints each tensor's name, shape and a checksum
 //
@@ -15,6 +17,7 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <random>
 
 static int inspect(const char *dir) {
     using namespace rllama;
@@ -47,6 +50,14 @@ int main(int argc, char **argv) {
             fprintf(stderr, "rllama_generate: %s\n", e.what());
             return 1;
         }
+    }
+    bool use_sampler = false;
+    rllama::TokenSampler sampler;
+    if (argc >= 6 && std::string(argv[1]) == "--sample") {
+        use_sampler = true;
+        sampler = sampler.top_k(strtoul(argv[2], nullptr, 10)).temperature(strtof(argv[3], nullptr)).top_p(strtof(argv[4], nullptr)).repetition_penalty(strtof(argv[5], nullptr));
+        argv += 5;
+        argc -= 5;
     }
     const char *model_path = nullptr;
     if (argc >= 3 && std::string(argv[1]) == "--model-path") {
@@ -91,7 +102,23 @@ int main(int argc, char **argv) {
         rlh_synth_tokens(seed, 0, n_prompt, 3, (int32_t)vocab, prompt.data());
         rllama::TransformerCaches caches = tr.make_caches();
         float ms_first = 0.0f, ms_tok = 0.0f;
-        std::vector<rllama::TokenId> out = tr.generate_greedy(prompt, n_new, caches, &ms_first, &ms_tok);
+        std::vector<rllama::TokenId> out;
+        if (!use_sampler) {
+            out = tr.generate_greedy(prompt, n_new, caches, &ms_first, &ms_tok);
+        } else { // the reference's loop: forward over the new tokens, sample with the tokens so far (src/rllama_main.rs:821-897)
+            std::mt19937 rng((uint32_t)seed);
+            std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+            std::vector<rllama::TokenId> toks = prompt, feed = prompt;
+            size_t pos = 0;
+            for (size_t i = 0; i < n_new; i++) {
+                auto [tok, prob] = tr.forward_sample(feed, pos, caches, sampler.raw(), toks, uni(rng));
+                (void)prob;
+                pos += feed.size();
+                feed.assign(1, tok);
+                toks.push_back(tok);
+                out.push_back(tok);
+            }
+        }
         printf("tokens:");
         for (rllama::TokenId t : out) printf(" %d", t);
         printf("\nTime taken to generate first token: %.0fms\n", ms_first);

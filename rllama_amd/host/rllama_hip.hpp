@@ -151,6 +151,15 @@ class Transformer {
         check(rlh_generate_greedy(h_, caches.raw(), prompt.data(), (int)prompt.size(), (int)n_new, out.data(), ms_first, ms_per_token));
         return out;
     }
+    // forward + TokenSampler::sample: the body of the token loop (src/rllama_main.rs:846-860)
+    std::pair<TokenId, float> forward_sample(const std::vector<TokenId> &tokens, size_t start_pos, TransformerCaches &caches, const rlh_sampler_params &sampler,
+                                             const std::vector<TokenId> &existing_tokens, float u) const {
+        TokenId tok = 0;
+        float prob = 0.0f;
+        check(rlh_forward_sample(h_, caches.raw(), tokens.data(), (int)tokens.size(), (int)start_pos, &sampler, existing_tokens.data(),
+                                 (int)existing_tokens.size(), u, &tok, &prob));
+        return {tok, prob};
+    }
     int last_layer_on_gpu() const { // src/transformer.rs:266-268
         int v = 0;
         check(rlh_model_layers_on_gpu(h_, &v));
@@ -162,6 +171,32 @@ class Transformer {
     std::shared_ptr<OpenCL> cl_;
     rlh_model *h_ = nullptr;
     size_t vocab_size_;
+};
+
+// TokenSampler (src/token_sampler.rs:6-174): builder-style settings; the arithmetic is the library's (host code).
+// The uniform variate of the draw comes from the caller (the reference uses rand::thread_rng).
+class TokenSampler {
+  public:
+    TokenSampler() { rlh_sampler_default(&p_); } // TokenSampler::new(), :20-29
+    TokenSampler temperature(float v) const { TokenSampler t = *this; t.p_.temperature = v; return t; }
+    TokenSampler top_p(float v) const { TokenSampler t = *this; t.p_.top_p = v; return t; }
+    TokenSampler top_k(size_t v) const { TokenSampler t = *this; t.p_.top_k = v > 0x7fffffffu ? 0x7fffffff : (int32_t)v; return t; }
+    TokenSampler repetition_penalty(float v) const { TokenSampler t = *this; t.p_.repetition_penalty = v; return t; }
+    float get_temperature() const { return p_.temperature; }
+    float get_top_p() const { return p_.top_p; }
+    size_t get_top_k() const { return (size_t)p_.top_k; }
+    float get_repetition_penalty() const { return p_.repetition_penalty; }
+    // sample(logits, tokenizer, existing_tokens) -> (token, probability) (:83-174); u in [0, 1]
+    std::pair<TokenId, float> sample(const std::vector<float> &logits, const std::vector<TokenId> &existing_tokens, float u) const {
+        TokenId tok = 0;
+        float prob = 0.0f;
+        check(rlh_sample(logits.data(), (int)logits.size(), &p_, existing_tokens.data(), (int)existing_tokens.size(), u, &tok, &prob));
+        return {tok, prob};
+    }
+    const rlh_sampler_params &raw() const { return p_; }
+
+  private:
+    rlh_sampler_params p_;
 };
 
 // Device tensor with the op set of OpenCLTensor (src/tensor_opencl_support.rs:215-405)

@@ -428,3 +428,32 @@ def test_model_loaded_from_checkpoint_directory(ctx, tmp_path, shards):
     assert r.returncode == 0, r.stderr
     line = [ln for ln in r.stdout.splitlines() if ln.startswith("tokens:")][0]
     assert [int(t) for t in line.split()[1:]] == [int(t) for t in want_ids]
+
+
+def test_forward_sample(ctx):
+    """rlh_forward_sample = forward + TokenSampler::sample (src/rllama_main.rs:846-860): with top_k 1 it is the device argmax,
+    otherwise the host sampler on the downloaded logits; both agree with the oracle sampler run on these logits."""
+    shape = SMALL
+    W = synth_weights(shape, seed=61, std=0.08, norm_ones=False)
+    gm = make_gpu(ctx, shape, W, True)
+    toks = np.random.default_rng(62).integers(0, shape.vocab_size, 7)
+
+    class _U:
+        def __init__(self, u):
+            self.u = u
+
+        def random(self, dtype=None):
+            return np.float32(self.u)
+
+    logits = gm.forward(toks, 0, gm.make_caches())
+    greedy = gm.forward_greedy(toks, 0, gm.make_caches())
+    for ts in (rllama_amd.TokenSampler(), rllama_amd.TokenSampler().temperature(3.0).repetition_penalty(1.0)):
+        tok, prob = gm.forward_sample(toks, 0, gm.make_caches(), ts, toks, _U(0.4))
+        oi, op, ot = oracle.sample_candidates(logits, ts.get_temperature(), ts.get_top_p(), ts.get_top_k(), ts.get_repetition_penalty(), toks)
+        assert tok == greedy == oi[0] and prob == 1.0
+    ts = rllama_amd.TokenSampler().temperature(1.5).top_k(8).top_p(0.9).repetition_penalty(1.2)
+    for u in (0.0, 0.35, 0.8, 1.0):
+        tok, prob = gm.forward_sample(toks, 0, gm.make_caches(), ts, toks, _U(u))
+        oi, op, ot = oracle.sample_candidates(logits, 1.5, 0.9, 8, 1.2, toks)
+        assert (tok, prob) == oracle.sample_pick(oi, op, ot, u)
+    gm.free()
