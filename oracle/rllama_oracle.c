@@ -22,9 +22,12 @@
  *                                   matmuls; invariants (prefill(n) == prefill(n-1)+decode(1), zeroed wo/w2
  *                                   closed form, true_clone determinism).
  *   greedy sampler                  brute-force restatement in Python on small vocabularies.
+ *   full sampler (candidates, pick) float64 closed form derived by hand from token_sampler.rs:99-159 (token 0 ends at exactly 0,
+ *                                   nothing else is shifted), token-0-only penalty, NaN-last ordering on overflow, agreement with
+ *                                   the greedy entry at top_k 1, frequency check of the cumulative walk over 20000 draws.
  *
  * parity unpinned (only a run of the real binary could pin them; none changes a tolerance-based check):
- *   - tie-break among exactly equal top probabilities (token_sampler.rs:131-145 uses sort_unstable_by);
+ *   - tie-break among exactly equal probabilities, greedy and full sampler alike (token_sampler.rs:131-145 uses sort_unstable_by);
  *   - whether LLVM folded powf(x, 2.0) to x*x in Tensor::pow (tensor.rs:537-547): at most 1 ulp per term,
  *     this file uses x*x;
  *   - num-complex's Complex::from_polar(1.0, t) == (cos t, sin t) (transformer.rs:880), taken from its docs.
