@@ -76,7 +76,7 @@ HOST_BIN = os.path.join(HERE, "host", "rllama_generate")
 def build_host(force: bool = False) -> str:
     """Compiles the C++ host example (header-only mirror of the reference API + the token loop) against the library."""
     src = os.path.join(HERE, "host", "generate_main.cpp")
-    hdrs = [os.path.join(HERE, "host", "rllama_hip.hpp"), os.path.join(HERE, "host", "model_files.hpp")]
+    hdrs = [os.path.join(HERE, "host", "rllama_hip.hpp"), os.path.join(HERE, "host", "model_files.hpp"), os.path.join(HERE, "host", "tokenizer.hpp")]
     if not force and os.path.exists(HOST_BIN) and all(os.path.getmtime(HOST_BIN) >= os.path.getmtime(f) for f in (src, *hdrs, LIB)):
         return HOST_BIN
     cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-Wextra", src, "-o", HOST_BIN, "-L" + HERE, "-lrllama_hip", "-Wl,-rpath,$ORIGIN/.."]

@@ -101,7 +101,10 @@ __device__ __forceinline__ float wave_sum_lane63(float v) {
 }
 
 constexpr int kGemvBurst = RLH_GEMV_BURST; // 16-byte loads per lane issued back to back before they are consumed
-constexpr int kGemvPrologueVecs = 8; // float4 loads per thread per prologue batch (one batch covers k <= 8192)
+#ifndef RLH_GEMV_PROLOGUE_VECS
+#define RLH_GEMV_PROLOGUE_VECS 8
+#endif
+constexpr int kGemvPrologueVecs = RLH_GEMV_PROLOGUE_VECS; // float4 loads per thread per prologue batch (one batch covers k <= 1024 * this)
 
 template <typename WT, typename XT, int kEpi, bool kStream>
 __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {

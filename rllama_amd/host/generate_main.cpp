@@ -7,6 +7,8 @@
 //                                                                 src/rllama_main.rs:44-45); prompt ids are synthetic
 //   ... --sample TOP_K TEMPERATURE TOP_P REPETITION_PENALTY      (before the other arguments) token loop with
 //                                                                 TokenSampler instead of the device-resident greedy loop
+//   rllama_generate --tokenize TOKENIZER_MODEL TEXT              no device needed: prints the ids of Tokenizer::tokenize_to_ids
+//                                                                 and the pieces (src/tokenizer.rs:127-177)
 //   rllama_generate --inspect DIR                                 no device needed: parses params.json and every data.pkl
 //                                                                 and prints each tensor's name, shape and a checksum
 //
@@ -14,6 +16,7 @@
 // the C ABI.  Exits non-zero with the library's message if there is no gfx950 device.
 #include "model_files.hpp"
 #include "rllama_hip.hpp"
+#include "tokenizer.hpp"
 
 #include <cstdio>
 #include <cstdlib>
@@ -46,6 +49,20 @@ int main(int argc, char **argv) {
     if (argc >= 3 && std::string(argv[1]) == "--inspect") {
         try {
             return inspect(argv[2]);
+        } catch (const std::exception &e) {
+            fprintf(stderr, "rllama_generate: %s\n", e.what());
+            return 1;
+        }
+    }
+    if (argc >= 4 && std::string(argv[1]) == "--tokenize") {
+        try {
+            const rllama::Tokenizer tok = rllama::Tokenizer::load(argv[2]);
+            printf("ids:");
+            for (rllama::TokenId t : tok.tokenize_to_ids(argv[3])) printf(" %d", t);
+            printf("\n");
+            for (rllama::TokenId t : tok.tokenize_to_ids(argv[3]))
+                if (t != 1) printf("piece %d %s\n", t, tok.id_to_str(t).c_str());
+            return 0;
         } catch (const std::exception &e) {
             fprintf(stderr, "rllama_generate: %s\n", e.what());
             return 1;
