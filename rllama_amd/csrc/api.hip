@@ -118,6 +118,8 @@ struct rlh_model {
     int stream_weights = 1;
     PrefillScratch pf;
     int prefill_mode = 0; // 0: matrix-core prefill where available (f16 mode), 1: token by token
+    // fused attention kernel for multi-token calls (head_dim 64 / 128); RLLAMA_HIP_PREFILL_ATTN=gemm keeps the two-GEMM path
+    bool prefill_attn_fused = !(getenv("RLLAMA_HIP_PREFILL_ATTN") && !strcmp(getenv("RLLAMA_HIP_PREFILL_ATTN"), "gemm"));
     // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
     int next_pos = -1;
     rlh_caches *greedy_caches = nullptr;
@@ -871,49 +873,66 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         rp.max_seq_len = P.max_seq_len;
         rp.t_pad = tp;
         HIP_TRY(launch_rope_kv_prefill(rp, st));
-        // scores[h] = q[h] . K[h]^T summed over the hi and lo parts of q: one pass that skips the tiles above the
-        // diagonal where the fast GEMM takes head_dim as a K segment, else one accumulating pass per part
-        const bool one_pass = hd % 64 == 0;
-        for (int part = 0; part < (one_pass ? 1 : 2); part++) {
-            GemmParams g{};
-            g.a = (const _Float16 *)S.q2 + (size_t)part * hd;
-            g.b = (const _Float16 *)ck;
-            g.c = S.scores;
-            g.m = n;
-            g.n = n;
-            g.k = one_pass ? 2 * hd : hd;
-            g.k_seg = one_pass ? hd : 0;
-            g.causal = one_pass ? 1 : 0;
-            g.accumulate = part;
-            g.lda = 2 * hd;
-            g.ldb = hd;
-            g.ldc = tp;
-            g.batch = H;
-            g.stride_a = (size_t)n * 2 * hd;
-            g.stride_b = (size_t)P.max_seq_len * hd;
-            g.stride_c = (size_t)n * tp;
-            HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
-        }
-        HIP_TRY(launch_causal_softmax(S.scores, S.p2, (char *)S.p2 + (size_t)tp * 2, H, n, tp, 2 * tp, hd, st));
-        {   // out[h] = P[h] . V[h] summed over the hi and lo parts of P, rounded to f16 and written as columns
-            // h * hd .. of the [n x dim] input of wo (the concat of heads and the rounding point of transformer.rs:783-796)
-            GemmParams g{};
-            g.a = (const _Float16 *)S.p2;
-            g.b = (const _Float16 *)S.v_t;
-            g.c = S.a;
-            g.m = n;
-            g.n = hd;
-            g.k = 2 * tp;
-            g.k_seg = tp;
-            g.causal = 2;
-            g.lda = 2 * tp;
-            g.ldb = tp;
-            g.ldc = d;
-            g.batch = H;
-            g.stride_a = (size_t)n * 2 * tp;
-            g.stride_b = (size_t)hd * tp;
-            g.stride_c = (size_t)hd;
-            HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
+        if (m->prefill_attn_fused && attn_prefill_supported(hd)) {
+            // scores, mask, softmax and P.V in one kernel; the score matrix never reaches memory
+            AttnPrefillParams ap{};
+            ap.q2 = S.q2;
+            ap.cache_k = ck;
+            ap.v_t = S.v_t;
+            ap.out = S.a;
+            ap.n = n;
+            ap.n_heads = H;
+            ap.head_dim = hd;
+            ap.dim = d;
+            ap.max_seq_len = P.max_seq_len;
+            ap.t_pad = tp;
+            ap.scale = 1.0f / sqrtf((float)hd);
+            HIP_TRY(launch_attn_prefill(ap, st));
+        } else {
+            // scores[h] = q[h] . K[h]^T summed over the hi and lo parts of q: one pass that skips the tiles above the
+            // diagonal where the fast GEMM takes head_dim as a K segment, else one accumulating pass per part
+            const bool one_pass = hd % 64 == 0;
+            for (int part = 0; part < (one_pass ? 1 : 2); part++) {
+                GemmParams g{};
+                g.a = (const _Float16 *)S.q2 + (size_t)part * hd;
+                g.b = (const _Float16 *)ck;
+                g.c = S.scores;
+                g.m = n;
+                g.n = n;
+                g.k = one_pass ? 2 * hd : hd;
+                g.k_seg = one_pass ? hd : 0;
+                g.causal = one_pass ? 1 : 0;
+                g.accumulate = part;
+                g.lda = 2 * hd;
+                g.ldb = hd;
+                g.ldc = tp;
+                g.batch = H;
+                g.stride_a = (size_t)n * 2 * hd;
+                g.stride_b = (size_t)P.max_seq_len * hd;
+                g.stride_c = (size_t)n * tp;
+                HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
+            }
+            HIP_TRY(launch_causal_softmax(S.scores, S.p2, (char *)S.p2 + (size_t)tp * 2, H, n, tp, 2 * tp, hd, st));
+            {   // out[h] = P[h] . V[h] summed over the hi and lo parts of P, rounded to f16 and written as columns
+                // h * hd .. of the [n x dim] input of wo (the concat of heads and the rounding point of transformer.rs:783-796)
+                GemmParams g{};
+                g.a = (const _Float16 *)S.p2;
+                g.b = (const _Float16 *)S.v_t;
+                g.c = S.a;
+                g.m = n;
+                g.n = hd;
+                g.k = 2 * tp;
+                g.k_seg = tp;
+                g.causal = 2;
+                g.lda = 2 * tp;
+                g.ldb = tp;
+                g.ldc = d;
+                g.batch = H;
+                g.stride_a = (size_t)n * 2 * tp;
+                g.stride_b = (size_t)hd * tp;
+                g.stride_c = (size_t)hd;
+                HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
+            }
         }
         if ((rc = gemm(S.a, d, L.wo.p, d, S.h, d, n, d, d, kGemmEpiResAddF32, S.x)) != RLH_OK) return rc;     // h = x + wo(att)
         HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.h, (const float *)L.ffn_norm.p, n, d, eps, st));

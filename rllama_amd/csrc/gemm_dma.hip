@@ -115,6 +115,25 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+    // Residual epilogue on small wavefront tiles: what the epilogue adds to is fetched now, before the K loop, so that its
+    // latency is gone by the time the accumulators are ready (these ordinary loads are older than every direct-to-LDS
+    // load below, so the hand-placed vmcnt waits only get stricter).  Each element is read and later written by the
+    // same lane, so C may alias the residual.
+    constexpr bool kEarlyResidual = kEpi == kGemmEpiResAddF32 && kNT <= 2;
+    [[maybe_unused]] float16_t early[kEarlyResidual ? 2 : 1][kEarlyResidual ? kNT : 1];
+    if constexpr (kEarlyResidual) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < kNT; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = bm0 + wm * 64 + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                    const int c = bn0 + wn * (32 * kNT) + j * 32 + (lane & 31);
+                    early[i][j][v] = (r < M && c < N) ? p.residual[(size_t)r * p.ldc + c] : 0.0f;
+                }
+    }
+
     // operand fragments: lane l supplies row (l % 32), logical chunk 2 * ks + l / 32 of a 32 x 16 slab
     const int frow = lane & 31, fch = lane >> 5;
     int a_off[2], a_sw[2], b_off[kNT], b_sw[kNT];
@@ -198,7 +217,10 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     for (int j = 0; j < kNT; j++) {
         const int c = out_col(j);
         [[maybe_unused]] float16_t prev[2];
-        if constexpr (kEpi != kGemmEpiF16) {
+        if constexpr (kEarlyResidual) {
+            prev[0] = early[0][j];
+            prev[1] = early[1][j];
+        } else if constexpr (kEpi != kGemmEpiF16) {
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll

@@ -112,6 +112,18 @@ struct PrefillRopeParams {
     int n, dim, head_dim, max_seq_len, t_pad;
     int q_stride;
 };
+// fused causal attention of a multi-token forward (attn_prefill.hip); head_dim 64 or 128, f16 cache
+struct AttnPrefillParams {
+    const void *q2;          // [n_heads][n] rows [q hi (head_dim) | q lo (head_dim)] f16, after RoPE
+    const void *cache_k;     // this layer: [n_heads][max_seq_len][head_dim] f16
+    const void *v_t;         // [n_heads][head_dim][t_pad] f16 (V transposed, finite values in the padding)
+    void *out;               // [n][dim] f16: head h at columns h * head_dim ..
+    int n, n_heads, head_dim, dim, max_seq_len, t_pad;
+    float scale;             // 1 / sqrt(head_dim) (transformer.rs:770)
+};
+bool attn_prefill_supported(int head_dim);
+hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s);
+
 hipError_t launch_embed_rows(const void *table, int table_f16, const int32_t *tokens_dev, int n, int dim, float *x, hipStream_t s);
 hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s);
 hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s);

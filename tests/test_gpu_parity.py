@@ -189,6 +189,23 @@ def test_forward_f16_mode(ctx, shape):
     gm.free()
 
 
+@pytest.mark.parametrize("n_heads,n", [(2, 300), (2, 129), (4, 64), (4, 1)], ids=["hd128-n300", "hd128-n129", "hd64-n64", "hd64-n1"])
+def test_prefill_fused_attention_head_dims(ctx, n_heads, n):
+    """The one-kernel causal attention of the multi-token forward (head_dim 128 and 64; ragged query and key tiles) against the oracle."""
+    shape = Shape(dim=256, n_layers=2, n_heads=n_heads, ffn_hidden=512, vocab_size=128, max_seq_len=320)
+    W = synth_weights(shape, seed=45, std=0.08, norm_ones=False)
+    toks = np.random.default_rng(46).integers(0, shape.vocab_size, n + 1)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    oc, gc = om.make_caches(), gm.make_caches()
+    m = max(n, 2)  # a 1-token call is a decode step; make it a 2-token prefill instead
+    want, got = om.forward(toks[:m], 0, oc), gm.forward(toks[:m], 0, gc)
+    assert max_rel_err(got, want) < TOL_F16, max_rel_err(got, want)
+    # and the step after it reads the cache the prefill wrote
+    want, got = om.forward(toks[m:m + 1], m, oc) if m < len(toks) else want, gm.forward(toks[m:m + 1], m, gc) if m < len(toks) else got
+    assert max_rel_err(got, want) < TOL_F16
+    gm.free()
+
+
 def test_prefill_long_prompt_causal_tiles(ctx):
     """A prompt long enough that the score matrix spans several GEMM tiles per head (tiles above the diagonal are
     skipped, the probability product stops at the diagonal) on the large-tile path; compared with the oracle."""
