@@ -1046,15 +1046,14 @@ extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *p
     CtxLock lock(m->ctx);
     hipStream_t st = m->ctx->stream;
     hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
-    HIP_TRY(hipEventCreate(&e2));
     auto cleanup = [&]() {
-        (void)hipEventDestroy(e0);
-        (void)hipEventDestroy(e1);
-        (void)hipEventDestroy(e2);
+        for (hipEvent_t ev : {e0, e1, e2})
+            if (ev) (void)hipEventDestroy(ev);
     };
-    hipError_t e = hipEventRecord(e0, st);
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess) e = hipEventCreate(&e2);
+    if (e == hipSuccess) e = hipEventRecord(e0, st);
     if (e == hipSuccess) {
         rc = enqueue_forward(m, c, prompt, n_prompt, 0);
         if (rc == RLH_OK) e = launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st);
