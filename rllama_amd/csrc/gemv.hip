@@ -101,6 +101,9 @@ __device__ __forceinline__ float wave_sum_lane63(float v) {
 }
 
 constexpr int kGemvBurst = RLH_GEMV_BURST; // 16-byte loads per lane issued back to back before they are consumed
+#ifndef RLH_GEMV_PRELOAD
+#define RLH_GEMV_PRELOAD 1
+#endif
 #ifndef RLH_GEMV_PROLOGUE_VECS
 #define RLH_GEMV_PROLOGUE_VECS 8
 #endif
@@ -126,6 +129,28 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     const int pieces_full = K / kPiece;
     const int kpad = pieces * kPiece;
 
+    // The first burst of this wavefront's first row unit does not depend on x: it is issued right behind the prologue's own
+    // loads (which stay ahead of it in the in-order return queue), so that its memory latency runs under the norm / staging work.
+    const WT *wmat[kMats];
+    wmat[0] = reinterpret_cast<const WT *>(p.w);
+    if constexpr (kMats == 2) wmat[1] = reinterpret_cast<const WT *>(p.w_b);
+    const int unit_first = blockIdx.x * kGemvWaves + wave;
+    // (measured: worth 1 % on the w1|w3 product, nothing or a loss on the others, so only that instantiation does it)
+    const bool have_pre = RLH_GEMV_PRELOAD && kEpi == kEpiSilu && unit_first < p.n_rows / kRows && kU <= pieces_full;
+    uint4_t wpre[kU][kMats][kRows];
+    auto preload = [&]() {
+        if (have_pre) {
+#pragma unroll
+            for (int u = 0; u < kU; u++)
+#pragma unroll
+                for (int m = 0; m < kMats; m++)
+#pragma unroll
+                    for (int r = 0; r < kRows; r++)
+                        wpre[u][m][r] = load16<kStream>(wmat[m] + (size_t)(unit_first * kRows + r) * K + (size_t)u * kPiece + lane * kVec);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
     // ---- prologue: x = (x_in [+ x_add]) [RMSNorm] [-> f16], staged in LDS, zero padded to kpad ----
     // All global loads of a batch are issued before any is consumed (one exposed memory latency per batch).
     const bool writes_sum = (p.x_out != nullptr) && blockIdx.x == 0;
@@ -146,6 +171,8 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
         }
 #pragma unroll
         for (int j = 0; j < kGemvPrologueVecs; j++) wv[j] = w4[min(tid + j * kGemvThreads, n4 - 1)];
+        __builtin_amdgcn_sched_barrier(0);
+        preload();
         float ss = 0.0f;
 #pragma unroll
         for (int j = 0; j < kGemvPrologueVecs; j++) {
@@ -168,6 +195,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
         }
     } else if (p.norm_w != nullptr) {
         // k too large for the register path: two passes over global memory
+        preload();
         float ss = 0.0f;
         for (int i = tid; i < K; i += kGemvThreads) {
             float v = p.x[i];
@@ -190,6 +218,10 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
             if (a4 != nullptr) {
 #pragma unroll
                 for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + a4[min(base + tid + j * kGemvThreads, n4 - 1)];
+            }
+            if (base == 0) {
+                __builtin_amdgcn_sched_barrier(0);
+                preload();
             }
 #pragma unroll
             for (int j = 0; j < kGemvPrologueVecs; j++) {
@@ -214,11 +246,8 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     //      grid reads one dense window of the matrix ----
     const int n_units = p.n_rows / kRows; // n_rows is a multiple of kRows (checked on the host)
     const int W = gridDim.x * kGemvWaves;
-    const WT *wmat[kMats];
-    wmat[0] = reinterpret_cast<const WT *>(p.w);
-    if constexpr (kMats == 2) wmat[1] = reinterpret_cast<const WT *>(p.w_b);
 
-    for (int unit = blockIdx.x * kGemvWaves + wave; unit < n_units; unit += W) {
+    for (int unit = unit_first; unit < n_units; unit += W) {
         const int row0 = unit * kRows;
         float acc[kMats][kRows];
 #pragma unroll
@@ -228,7 +257,14 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
 
         for (int c = 0; c < pieces; c += kU) {
             uint4_t wv[kU][kMats][kRows];
-            if (c + kU <= pieces_full) {
+            if (have_pre && c == 0 && unit == unit_first) {
+#pragma unroll
+                for (int u = 0; u < kU; u++)
+#pragma unroll
+                    for (int m = 0; m < kMats; m++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[u][m][r];
+            } else if (c + kU <= pieces_full) {
                 // full burst: addresses differ by compile-time offsets
 #pragma unroll
                 for (int u = 0; u < kU; u++)
