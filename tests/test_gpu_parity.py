@@ -258,6 +258,20 @@ def test_long_context_split_attention(ctx):
         gm.free()
 
 
+def test_very_long_context_capped_splits(ctx):
+    """Positions beyond (splits cap) x (chunk): every attention block takes a longer share; also a 4300-token prompt through
+    the one-kernel prefill attention (68 key tiles) and the KV cache it leaves.  f16 mode, head_dim 64."""
+    shape = Shape(dim=128, n_layers=1, n_heads=2, ffn_hidden=256, vocab_size=200, max_seq_len=4400)
+    W = synth_weights(shape, seed=29, std=0.1, norm_ones=False)
+    toks = np.random.default_rng(30).integers(0, shape.vocab_size, 4320)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    oc, gc = om.make_caches(), gm.make_caches()
+    assert max_rel_err(gm.forward(toks[:4300], 0, gc), om.forward(toks[:4300], 0, oc)) < TOL_F16
+    for i in range(4300, 4320):
+        assert max_rel_err(gm.forward(toks[i:i + 1], i, gc), om.forward(toks[i:i + 1], i, oc)) < TOL_F16, i
+    gm.free()
+
+
 def test_config0_greedy_tokens_identical(ctx):
     """Config 0: d=1024, L=8, H=16, F=2816, V=32000, f16, seed 0; 16 prompt ids, then 64 greedy steps."""
     shape = CONFIG0
