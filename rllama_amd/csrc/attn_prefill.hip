@@ -111,7 +111,10 @@ __global__ __launch_bounds__(kApThreads) void attn_prefill_kernel(AttnPrefillPar
         for (int i = 0; i < kVLoads; i++) {
             const int c = tid + i * kApThreads;
             const int row = c / 8, ch = c % 8;
-            *reinterpret_cast<uint4_t *>(lds_v + row * kVRowBytes + ((ch ^ ((row >> 1) & 7)) << 4)) = vreg[i];
+            // rows with bit 4 set keep the two 8-byte halves of every chunk swapped: a half-wave reads one 8-byte half per
+            // row of 32 consecutive rows, and rows r and r + 16 would otherwise meet in the same banks
+            const uint4_t vv = (row & 16) ? uint4_t{vreg[i][2], vreg[i][3], vreg[i][0], vreg[i][1]} : vreg[i];
+            *reinterpret_cast<uint4_t *>(lds_v + row * kVRowBytes + ((ch ^ ((row >> 1) & 7)) << 4)) = vv;
         }
     };
 
@@ -193,8 +196,9 @@ __global__ __launch_bounds__(kApThreads) void attn_prefill_kernel(AttnPrefillPar
                     const int vrow = d * 32 + col;
                     const unsigned char *rowp = lds_v + vrow * kVRowBytes;
                     const int sw = (vrow >> 1) & 7;
-                    const half4_t a0 = *reinterpret_cast<const half4_t *>(rowp + ((((kk) >> 3) ^ sw) << 4) + ((kk & 4) << 1));
-                    const half4_t a1 = *reinterpret_cast<const half4_t *>(rowp + ((((kk + 8) >> 3) ^ sw) << 4) + ((kk & 4) << 1));
+                    const int sub = (((kk & 4) << 1)) ^ ((vrow & 16) >> 1); // which 8-byte half of the chunk (halves swapped in rows with bit 4 set)
+                    const half4_t a0 = *reinterpret_cast<const half4_t *>(rowp + ((((kk) >> 3) ^ sw) << 4) + sub);
+                    const half4_t a1 = *reinterpret_cast<const half4_t *>(rowp + ((((kk + 8) >> 3) ^ sw) << 4) + sub);
                     half8_t vf;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
