@@ -5,7 +5,8 @@
 // Numerics.  The reference keeps q (after RoPE) and the probabilities in fp32 and multiplies them with f16 K / V
 // widened to fp32.  Here q and P are split into hi + lo f16 halves and both halves go through the MFMA, accumulated in
 // fp32, so no rounding point is added; the softmax is evaluated in its streaming form (running maximum m, running sum l,
-// rescaled accumulator), which is the same function as exp(s) / sum exp(s) wherever that is finite.  The output is
+// rescaled accumulator; exponentials through exp2), which is the same function as exp(s) / sum exp(s) wherever that is
+// finite.  The output is
 // rounded to f16 where the reference does (transformer.rs:793-796).
 //
 // Blocking.  Workgroup = 4 wavefronts = 128 queries of one head; a wavefront owns 32 queries and walks the keys in
@@ -144,36 +145,49 @@ __global__ __launch_bounds__(kApThreads) void attn_prefill_kernel(AttnPrefillPar
                 }
             }
         }
-        // ---- scale (transformer.rs:768-770), causal mask (tensor.rs:496-508: col >= row + 1 is -inf), streaming softmax
+        // ---- scale (transformer.rs:768-770), causal mask (tensor.rs:496-508: col >= row + 1 is -inf), streaming softmax.
+        //      The vector ALU is what this kernel waits for, so the work per score is kept small: the maximum is taken on
+        //      the raw scores (the scale is positive), scale and log2(e) are folded into one multiplier of an exp2
+        //      (exp(scale s - scale m) = exp2(c s - c m), one fused multiply-add and one v_exp_f32 per score; the
+        //      argument error is a few 1e-6 relative in the probability), the mask is applied only on tiles that reach
+        //      the diagonal, and the accumulator is rescaled only when some row's maximum moved.
+        if (key0 + kApKeys - 1 > q0) { // some key of the tile lies after some query of this wavefront
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int key = key0 + j * 32 + (v >> 2) * 8 + half * 4 + (v & 3);
+                    if (key > my_q) s_acc[j][v] = -INFINITY;
+                }
+        }
         float m_tile = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int key = key0 + j * 32 + (v >> 2) * 8 + half * 4 + (v & 3);
-                const float s = key <= my_q ? s_acc[j][v] * p.scale : -INFINITY;
-                s_acc[j][v] = s;
-                m_tile = fmaxf(m_tile, s);
-            }
+            for (int v = 0; v < 16; v++) m_tile = fmaxf(m_tile, s_acc[j][v]);
         m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
         // the tile holds at least key0 <= q0 <= my_q, so m_tile is finite
+        const float c2 = p.scale * 1.44269504088896340736f;
         const float m_new = fmaxf(m_run, m_tile);
-        const float alpha = expf(m_run - m_new); // first tile: exp(-inf) = 0
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2); // first tile: exp2(-inf) = 0
         m_run = m_new;
+        const float mc = m_new * c2;
         float l_tile = 0.0f;
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const float e = expf(s_acc[j][v] - m_new); // masked: exp(-inf) = 0
+                const float e = __builtin_amdgcn_exp2f(fmaf(s_acc[j][v], c2, -mc)); // masked: exp2(-inf) = 0
                 s_acc[j][v] = e;
                 l_tile += e;
             }
         l_run = l_run * alpha + l_tile; // this lane's half of the row; the halves are added at the end
+        if (!__all(alpha == 1.0f)) {
 #pragma unroll
-        for (int d = 0; d < kDT; d++)
+            for (int d = 0; d < kDT; d++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) o_acc[d][v] *= alpha;
+                for (int v = 0; v < 16; v++) o_acc[d][v] *= alpha;
+        }
 
         // ---- O^T += V^T . P, probabilities split hi + lo.  k slot i of lane half h in 16-slot slab s of group j is key
         //      32 j + 16 s + 8 (i / 4) + 4 h + i % 4: the order the accumulator holds them in
