@@ -26,16 +26,48 @@ hipError_t launch_embed_rows(const void *table, int table_f16, const int32_t *to
     return hipGetLastError();
 }
 
-// RMSNorm::forward per row (transformer.rs:476-480), output rounded to f16 for the projections that follow
+// RMSNorm::forward per row (transformer.rs:476-480), output rounded to f16 for the projections that follow.
+// One workgroup per row; rows of up to 256 x 4 x kNormVecs floats are read once (16-byte loads, kept in registers).
+constexpr int kNormVecs = 8;
 __global__ __launch_bounds__(256) void rmsnorm_rows_f16_kernel(half_t *y, const float *x, const float *w, int d, float eps) {
     __shared__ float red[16];
     const float *xr = x + (size_t)blockIdx.x * d;
     half_t *yr = y + (size_t)blockIdx.x * d;
+    const int tid = threadIdx.x;
+    if ((d & 3) == 0 && d <= 256 * 4 * kNormVecs) {
+        const int n4 = d / 4;
+        const float4_t *x4 = reinterpret_cast<const float4_t *>(xr);
+        const float4_t *w4 = reinterpret_cast<const float4_t *>(w);
+        float4_t xv[kNormVecs];
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kNormVecs; j++) {
+            const int i = tid + j * 256;
+            xv[j] = i < n4 ? x4[i] : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int e = 0; e < 4; e++) ss = fmaf(xv[j][e], xv[j][e], ss);
+        }
+        ss = block_sum(ss, red);
+        const float rs = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+        for (int j = 0; j < kNormVecs; j++) {
+            const int i = tid + j * 256;
+            if (i < n4) {
+                const float4_t wv = w4[i];
+                typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
+                half4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = (half_t)((xv[j][e] * rs) * wv[e]);
+                *reinterpret_cast<half4_t *>(yr + i * 4) = o;
+            }
+        }
+        return;
+    }
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
+    for (int i = tid; i < d; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
     ss = block_sum(ss, red);
     const float rs = 1.0f / sqrtf(ss / (float)d + eps);
-    for (int i = threadIdx.x; i < d; i += blockDim.x) yr[i] = (half_t)((xr[i] * rs) * w[i]);
+    for (int i = tid; i < d; i += blockDim.x) yr[i] = (half_t)((xr[i] * rs) * w[i]);
 }
 
 hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s) {
@@ -93,7 +125,69 @@ __global__ void rope_kv_prefill_kernel(PrefillRopeParams p) {
     }
 }
 
+// The same for f16 caches, tiled: a workgroup takes 64 positions of one head, moves everything in 16-byte pieces (8 dims = 4
+// RoPE pairs of one row per thread and step) and transposes V through LDS so that V^T is written in 128-byte rows too.
+constexpr int kRopeTileRows = 64;
+__global__ __launch_bounds__(256) void rope_kv_prefill_tiled_kernel(PrefillRopeParams p) {
+    typedef __attribute__((ext_vector_type(8))) _Float16 h8;
+    constexpr int kPad = kRopeTileRows + 8; // halves per LDS row of the transposed V tile
+    __shared__ __attribute__((aligned(16))) half_t vt_tile[128 * kPad];
+    const int hd = p.head_dim, half_hd = hd / 2;
+    const int head = blockIdx.y, r0 = blockIdx.x * kRopeTileRows;
+    const int chunks = hd / 8; // 16-byte pieces per row
+    const half_t *qkv = reinterpret_cast<const half_t *>(p.qkv);
+    half_t *qhi = reinterpret_cast<half_t *>(p.q_hi), *qlo = reinterpret_cast<half_t *>(p.q_lo);
+    half_t *ck = reinterpret_cast<half_t *>(p.cache_k), *cv = reinterpret_cast<half_t *>(p.cache_v);
+    for (int c = threadIdx.x; c < kRopeTileRows * chunks; c += blockDim.x) {
+        const int rr = c / chunks, ch = c - rr * chunks;
+        const int r = r0 + rr;
+        const int j = head * hd + ch * 8; // first of this piece's 8 dims within the row of q / k / v
+        h8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (r < p.n) {
+            const half_t *row = qkv + (size_t)r * 3 * p.dim;
+            const h8 q8 = *reinterpret_cast<const h8 *>(row + j);
+            const h8 k8 = *reinterpret_cast<const h8 *>(row + p.dim + j);
+            v8 = *reinterpret_cast<const h8 *>(row + 2 * p.dim + j);
+            const float2 *fr = p.freqs + (size_t)r * half_hd + ch * 4;
+            h8 qh, ql, kk;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float2 f = fr[e];
+                float a, b;
+                rope_pair((float)q8[2 * e], (float)q8[2 * e + 1], f, a, b);
+                const half_t ah = (half_t)a, bh = (half_t)b;
+                qh[2 * e] = ah;
+                qh[2 * e + 1] = bh;
+                ql[2 * e] = (half_t)(a - (float)ah);
+                ql[2 * e + 1] = (half_t)(b - (float)bh);
+                rope_pair((float)k8[2 * e], (float)k8[2 * e + 1], f, a, b);
+                kk[2 * e] = (half_t)a; // Tensor::set_f32 on an f16 cache (tensor.rs:373-376)
+                kk[2 * e + 1] = (half_t)b;
+            }
+            const size_t qo = ((size_t)head * p.n + r) * p.q_stride + ch * 8;
+            *reinterpret_cast<h8 *>(qhi + qo) = qh;
+            *reinterpret_cast<h8 *>(qlo + qo) = ql;
+            const size_t co = ((size_t)head * p.max_seq_len + r) * hd + ch * 8;
+            *reinterpret_cast<h8 *>(ck + co) = kk;
+            *reinterpret_cast<h8 *>(cv + co) = v8;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) vt_tile[(ch * 8 + e) * kPad + rr] = v8[e]; // zeros for positions past n: finite padding
+    }
+    __syncthreads();
+    half_t *vt = reinterpret_cast<half_t *>(p.v_t) + (size_t)head * hd * p.t_pad + r0;
+    for (int c = threadIdx.x; c < hd * (kRopeTileRows / 8); c += blockDim.x) {
+        const int jrow = c / (kRopeTileRows / 8), ch = c - jrow * (kRopeTileRows / 8);
+        *reinterpret_cast<h8 *>(vt + (size_t)jrow * p.t_pad + ch * 8) = *reinterpret_cast<const h8 *>(&vt_tile[jrow * kPad + ch * 8]);
+    }
+}
+
 hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s) {
+    if (p.cache_f16 && p.head_dim % 8 == 0 && p.head_dim <= 128 && p.t_pad % kRopeTileRows == 0 && p.q_stride % 8 == 0 && p.dim % 8 == 0) {
+        const int n_heads = p.dim / p.head_dim;
+        hipLaunchKernelGGL(rope_kv_prefill_tiled_kernel, dim3((p.n + kRopeTileRows - 1) / kRopeTileRows, n_heads), dim3(256), 0, s, p);
+        return hipGetLastError();
+    }
     const size_t total = (size_t)p.n * (p.dim / 2);
     const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
     hipLaunchKernelGGL(rope_kv_prefill_kernel, dim3(blocks), dim3(256), 0, s, p);
@@ -161,19 +255,32 @@ hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, in
     return hipGetLastError();
 }
 
-// m = f16r(silu(g) * u) on f16 tensors (transformer.rs:557-565; tensor.rs:822-832, 722-734)
+// m = f16r(silu(g) * u) on f16 tensors (transformer.rs:557-565; tensor.rs:822-832, 722-734), 8 elements per thread
 __global__ void silu_mul_f16_kernel(const half_t *g, const half_t *u, half_t *m, size_t total) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const float gv = (float)g[i];
-        const float sg = gv / (1.0f + expf(-gv));
+    const size_t n8 = total / 8;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
+        const half8_t gv = reinterpret_cast<const half8_t *>(g)[i], uv = reinterpret_cast<const half8_t *>(u)[i];
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float x = (float)gv[e];
+            const float sg = x / (1.0f + expf(-x));
+            o[e] = (half_t)(sg * (float)uv[e]);
+        }
+        reinterpret_cast<half8_t *>(m)[i] = o;
+    }
+    for (size_t i = n8 * 8 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const float x = (float)g[i];
+        const float sg = x / (1.0f + expf(-x));
         m[i] = (half_t)(sg * (float)u[i]);
     }
 }
 
 hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s) {
-    const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
-    hipLaunchKernelGGL(silu_mul_f16_kernel, dim3(blocks), dim3(256), 0, s, (const half_t *)g, (const half_t *)u, (half_t *)m, total);
+    const size_t work = (total + 7) / 8;
+    const int blocks = (int)((work + 255) / 256 < 8192 ? (work + 255) / 256 : 8192);
+    hipLaunchKernelGGL(silu_mul_f16_kernel, dim3(blocks > 0 ? blocks : 1), dim3(256), 0, s, (const half_t *)g, (const half_t *)u, (half_t *)m, total);
     return hipGetLastError();
 }
 
