@@ -488,3 +488,33 @@ def test_forward_sample(ctx):
         oi, op, ot = oracle.sample_candidates(logits, 1.5, 0.9, 8, 1.2, toks)
         assert (tok, prob) == oracle.sample_pick(oi, op, ot, u)
     gm.free()
+
+
+def test_against_committed_oracle_fixtures(ctx):
+    """The committed outputs of the oracle (tests/golden/*.json; no oracle run here): config 0's 64 greedy ids identical,
+    its sampled logits and the tiny shapes' full logits within the f16 / f32 tolerances."""
+    import json
+    import os
+    gold = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    fx = json.load(open(os.path.join(gold, "config0_oracle.json")))
+    bits = lambda b: np.array(b, dtype=np.uint32).view(np.float32)  # noqa: E731
+    gm = make_gpu(ctx, CONFIG0, synth_weights(CONFIG0, seed=fx["seed"], std=fx["std"]), True)
+    ids, _, _ = gm.generate_greedy(fx["prompt_ids"], 64, gm.make_caches())
+    assert ids.tolist() == fx["greedy_ids"]
+    gc, toks, prev = gm.make_caches(), list(fx["prompt_ids"]), 0
+    for step in range(64):
+        lg = gm.forward(toks[prev:], prev, gc)
+        want = bits(fx["sample_logits_f32_bits"][step])
+        assert np.max(np.abs(lg[fx["sample_token_ids"]] - want)) <= TOL_F16 * np.max(np.abs(want)), step
+        toks.append(fx["greedy_ids"][step])
+        prev = len(toks) - 1
+    gm.free()
+    tiny = json.load(open(os.path.join(gold, "tiny_oracle.json")))
+    for mode, W, f16, tol in (("f16", synth_weights(TINY, seed=21, std=0.08, norm_ones=False), True, TOL_F16),
+                              ("f32", random_f32_weights(TINY, seed=23, std=0.08), False, TOL_F32)):
+        gm = make_gpu(ctx, TINY, W, f16)
+        gc = gm.make_caches()
+        t = tiny[mode]["tokens"]
+        assert max_rel_err(gm.forward(t[:7], 0, gc), bits(tiny[mode]["logits_after_7_f32_bits"])) < tol
+        assert max_rel_err(gm.forward(t[7:8], 7, gc), bits(tiny[mode]["logits_after_8_f32_bits"])) < tol
+        gm.free()

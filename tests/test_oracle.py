@@ -419,3 +419,52 @@ def test_cache_shift_left():
     T = shape.max_seq_len
     assert np.array_equal(after[:, : T - 2], before[:, 2:])
     assert np.array_equal(after[:, T - 2:], np.repeat(before[:, T - 1:], 2, axis=1))   # last column keeps its value
+
+
+# ---- committed fixtures (tests/golden/make_oracle_fixtures.py): the oracle must keep reproducing them -----------------
+
+def _bits_to_f32(bits):
+    return np.array(bits, dtype=np.uint32).view(np.float32)
+
+
+def test_golden_config0_reproduced():
+    import hashlib
+    import json
+    import os
+    import rllama_amd
+    from common import CONFIG0, make_oracle, synth_weights
+    fx = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config0_oracle.json")))
+    W = synth_weights(CONFIG0, seed=fx["seed"], std=fx["std"])
+    names = {rllama_amd.TOK_EMB: "tok_embeddings", rllama_amd.OUTPUT: "output", rllama_amd.WQ: "wq", rllama_amd.WK: "wk", rllama_amd.WV: "wv",
+             rllama_amd.WO: "wo", rllama_amd.W1: "w1", rllama_amd.W2: "w2", rllama_amd.W3: "w3"}
+    for (k, l), a in W.items():
+        if k in names:
+            assert hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest() == fx["weight_sha256"][f"{names[k]}.{l}"], (k, l)
+    prompt = rllama_amd.synth_tokens(0, 16, 3, 32000)
+    assert prompt.tolist() == fx["prompt_ids"]
+    om = make_oracle(CONFIG0, W, True)
+    oc = om.make_caches()
+    toks, prev = list(fx["prompt_ids"]), 0
+    for step in range(64):
+        logits = om.forward(toks[prev:], prev, oc)
+        tok, _, _ = oracle.sample_greedy(logits)
+        want = _bits_to_f32(fx["sample_logits_f32_bits"][step])
+        got = logits[fx["sample_token_ids"]]
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-7), step
+        assert tok == fx["greedy_ids"][step], step
+        toks.append(tok)
+        prev = len(toks) - 1
+    assert min(fx["top2_logit_gap"]) > 1e-4  # the greedy choice is nowhere near a tie, so f16-level noise cannot flip it
+
+
+def test_golden_tiny_reproduced():
+    import json
+    import os
+    from common import TINY, make_oracle, random_f32_weights, synth_weights
+    fx = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tiny_oracle.json")))
+    for mode, W, f16 in (("f16", synth_weights(TINY, seed=21, std=0.08, norm_ones=False), True), ("f32", random_f32_weights(TINY, seed=23, std=0.08), False)):
+        om = make_oracle(TINY, W, f16)
+        oc = om.make_caches()
+        toks = fx[mode]["tokens"]
+        assert np.allclose(om.forward(toks[:7], 0, oc), _bits_to_f32(fx[mode]["logits_after_7_f32_bits"]), rtol=1e-6, atol=1e-7)
+        assert np.allclose(om.forward(toks[7:8], 7, oc), _bits_to_f32(fx[mode]["logits_after_8_f32_bits"]), rtol=1e-6, atol=1e-7)
