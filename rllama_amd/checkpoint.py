@@ -426,3 +426,44 @@ def write_checkpoint(model_path: str, params: dict, tensors: Dict[str, np.ndarra
             entries.append((name, str(k), tuple(int(v) for v in piece.shape)))
         with open(os.path.join(sd, "data.pkl"), "wb") as f:
             f.write(pickle_state_dict(entries))
+
+
+def write_synthetic_checkpoint(model_path: str, dim: int = 1024, n_layers: int = 8, n_heads: int = 16, ffn_hidden: int = 2816, vocab_size: int = 32000,
+                               norm_eps: float = 1e-6, seed: int = 0, std: float = 0.02, n_shards: int = 1) -> None:
+    """The benchmark's synthetic model (weights N(0, std) from the counter-based generator, norm weights 1.0) as a model
+    directory the reference can be pointed at (--model-path; it also wants a tokenizer model, which this does not make).
+    The defaults are config 0."""
+    import rllama_amd as ra
+
+    one = np.full(dim, 0x3C00, dtype=np.uint16)  # 1.0 in f16
+    T: Dict[str, np.ndarray] = {}
+
+    def gen(kind, layer, rows, cols):
+        return ra.synth_normal_f16(seed, kind, layer, rows * cols, std=std).reshape(rows, cols)
+
+    T["tok_embeddings.weight"] = gen(ra.TOK_EMB, 0, vocab_size, dim)
+    T["norm.weight"] = one
+    T["output.weight"] = gen(ra.OUTPUT, 0, vocab_size, dim)
+    for l in range(n_layers):
+        p = f"layers.{l}."
+        for nm, kind in (("attention.wq", ra.WQ), ("attention.wk", ra.WK), ("attention.wv", ra.WV), ("attention.wo", ra.WO)):
+            T[p + nm + ".weight"] = gen(kind, l, dim, dim)
+        T[p + "feed_forward.w1.weight"] = gen(ra.W1, l, ffn_hidden, dim)
+        T[p + "feed_forward.w2.weight"] = gen(ra.W2, l, dim, ffn_hidden)
+        T[p + "feed_forward.w3.weight"] = gen(ra.W3, l, ffn_hidden, dim)
+        T[p + "attention_norm.weight"] = one
+        T[p + "ffn_norm.weight"] = one
+    write_checkpoint(model_path, {"dim": dim, "multiple_of": 256, "n_heads": n_heads, "n_layers": n_layers, "norm_eps": norm_eps, "vocab_size": vocab_size},
+                     T, n_shards=n_shards)
+
+
+if __name__ == "__main__":
+    import argparse
+
+    ap = argparse.ArgumentParser(description="write the synthetic benchmark model (default: config 0) in the reference's on-disk layout")
+    ap.add_argument("model_path")
+    for name, default in (("dim", 1024), ("n-layers", 8), ("n-heads", 16), ("ffn-hidden", 2816), ("vocab-size", 32000), ("seed", 0), ("shards", 1)):
+        ap.add_argument("--" + name, type=int, default=default)
+    a = ap.parse_args()
+    write_synthetic_checkpoint(a.model_path, a.dim, a.n_layers, a.n_heads, a.ffn_hidden, a.vocab_size, seed=a.seed, n_shards=a.shards)
+    print("wrote", a.model_path)

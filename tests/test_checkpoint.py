@@ -242,3 +242,17 @@ def test_cpp_host_loader_reads_what_the_python_writer_wrote(tmp_path):
     # and the failure path: a directory without params.json
     r = subprocess.run([exe, "--inspect", str(tmp_path)], capture_output=True, text=True, timeout=60)
     assert r.returncode == 1 and "Unknown source" in r.stderr
+
+
+def test_synthetic_checkpoint_matches_the_generator(tmp_path):
+    """The benchmark model written to disk holds exactly the generator's bits (the weights every other test uses)."""
+    import rllama_amd
+    path = str(tmp_path / "syn")
+    ck.write_synthetic_checkpoint(path, dim=64, n_layers=2, n_heads=2, ffn_hidden=192, vocab_size=96, seed=3, n_shards=2)
+    c = ck.Checkpoint(path)
+    assert (c.dim, c.n_layers, c.n_heads, c.vocab_size, c.norm_eps) == (64, 2, 2, 96, 1e-6)
+    w2 = c.load_f16_bits("layers.1.feed_forward.w2.weight", ck.FROM_PIECES_COLS)
+    assert np.array_equal(w2, rllama_amd.synth_normal_f16(3, rllama_amd.W2, 1, 64 * 192).reshape(64, 192))
+    emb = c.load_f16_bits("tok_embeddings.weight", ck.FROM_PIECES_COLS)
+    assert np.array_equal(emb, rllama_amd.synth_normal_f16(3, rllama_amd.TOK_EMB, 0, 96 * 64).reshape(96, 64))
+    assert np.all(c.load_f16_bits("layers.0.ffn_norm.weight", ck.FROM_PIECES_ROWS, True) == 0x3C00)
