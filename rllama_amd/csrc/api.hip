@@ -120,6 +120,7 @@ struct rlh_model {
     int prefill_mode = 0; // 0: matrix-core prefill where available (f16 mode), 1: token by token
     // fused attention kernel for multi-token calls (head_dim 64 / 128); RLLAMA_HIP_PREFILL_ATTN=gemm keeps the two-GEMM path
     bool prefill_attn_fused = !(getenv("RLLAMA_HIP_PREFILL_ATTN") && !strcmp(getenv("RLLAMA_HIP_PREFILL_ATTN"), "gemm"));
+    int prefill_attn_order = getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER") ? atoi(getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER")) : 2;
     // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
     int next_pos = -1;
     rlh_caches *greedy_caches = nullptr;
@@ -872,8 +873,10 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         rp.head_dim = hd;
         rp.max_seq_len = P.max_seq_len;
         rp.t_pad = tp;
+        const bool fused = m->prefill_attn_fused && attn_prefill_supported(hd);
+        rp.vt_swap = fused ? 1 : 0;
         HIP_TRY(launch_rope_kv_prefill(rp, st));
-        if (m->prefill_attn_fused && attn_prefill_supported(hd)) {
+        if (fused) {
             // scores, mask, softmax and P.V in one kernel; the score matrix never reaches memory
             AttnPrefillParams ap{};
             ap.q2 = S.q2;
@@ -887,6 +890,7 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
             ap.max_seq_len = P.max_seq_len;
             ap.t_pad = tp;
             ap.scale = 1.0f / sqrtf((float)hd);
+            ap.order = m->prefill_attn_order;
             HIP_TRY(launch_attn_prefill(ap, st));
         } else {
             // scores[h] = q[h] . K[h]^T summed over the hi and lo parts of q: one pass that skips the tiles above the

@@ -6,20 +6,26 @@
 // widened to fp32.  Here q and P are split into hi + lo f16 halves and both halves go through the MFMA, accumulated in
 // fp32, so no rounding point is added; the softmax is evaluated in its streaming form (running maximum m, running sum l,
 // rescaled accumulator; exponentials through exp2), which is the same function as exp(s) / sum exp(s) wherever that is
-// finite.  The output is
-// rounded to f16 where the reference does (transformer.rs:793-796).
+// finite.  The output is rounded to f16 where the reference does (transformer.rs:793-796).
 //
-// Blocking.  Workgroup = 4 wavefronts = 128 queries of one head; a wavefront owns 32 queries and walks the keys in
-// tiles of 64 (K tile [64 x hd] and V^T tile [hd x 64] staged in LDS once for the four wavefronts, next tile's global
-// loads in flight while the current one is used).  Both products are computed transposed so that every per-query
-// quantity lives in one lane pair:
+// Blocking.  Workgroup = 4 wavefronts = 64 queries of one head.  Wavefront (g, h) owns the 32 queries of query group g
+// and, of every 64-key tile, the 32 keys of key half h; the two halves keep their own (m, l, O) and are merged through
+// LDS at the end.  Splitting the keys rather than taking more queries doubles the number of workgroups (two fit on a
+// compute unit, so every SIMD holds two wavefronts and one's softmax arithmetic overlaps the other's MFMAs) and lets
+// light and heavy query blocks (1 .. n / 64 key tiles, causal) share a compute unit.  The K tile [64 x hd] and the V^T
+// tile [hd x 64] go from global memory straight into LDS (global_load_lds, two stages: the next tile's loads are in
+// flight while the current one is used; one barrier per tile).
+//
+// Both products are computed transposed so that every per-query quantity lives in one lane pair:
 //   S^T [key x query]  = K (A operand, rows = keys)   x  q (B operand, rows = queries), summed over hd
 //   O^T [dim x query] += V^T (A operand, rows = dims)  x  P (B operand, rows = queries), summed over keys
 // With v_mfma_f32_32x32x16_f16 the accumulator register v of lane l holds row 8 (v / 4) + 4 (l / 32) + v % 4 and column
 // l % 32: the column is the query in both products, so max / sum / rescale need one exchange with lane l ^ 32 and no
 // other cross-lane traffic.  The 16 probabilities a lane holds for a 32-key group are exactly what it must supply as the
-// B operand of the second product if the k slots of that MFMA are assigned to keys in the accumulator's order; V^T is
-// read from LDS in the same order (two 8-byte reads per operand).
+// B operand of the second product if the k slots of that MFMA are assigned to keys in the accumulator's order: slot i
+// of lane half h in 16-key slab s is key 16 s + 8 (i / 4) + 4 h + i % 4.  V^T is stored with the keys of every 16-key
+// group in the order 0-3, 8-11, 4-7, 12-15 (bits 2 and 3 of the position swapped, see rope_kv_prefill_tiled_kernel), so
+// that the 8 keys of a lane half are one 16-byte piece.
 #include "kernels.h"
 #include "device_utils.h"
 
@@ -28,33 +34,54 @@ namespace rlh {
 typedef __attribute__((ext_vector_type(16))) float float16_t;
 typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
 
-constexpr int kApQueries = 128; // per workgroup
-constexpr int kApKeys = 64;     // per key tile
+constexpr int kApQueries = 64; // per workgroup
+constexpr int kApKeys = 64;    // per key tile
 constexpr int kApThreads = 256;
 
 template <int HD>
-__global__ __launch_bounds__(kApThreads) void attn_prefill_kernel(AttnPrefillParams p) {
-    constexpr int kKS = HD / 16;                 // MFMA K-steps over the head dimension
-    constexpr int kDT = HD / 32;                 // 32-row tiles of O^T
-    constexpr int kKRowBytes = HD * 2;           // K tile row (one key)
-    constexpr int kKChunks = HD / 8;             // 16-byte chunks per K row
+__global__ __launch_bounds__(kApThreads, 2) void attn_prefill_kernel(AttnPrefillParams p) {
+    constexpr int kKS = HD / 16;                  // MFMA K-steps over the head dimension
+    constexpr int kDT = HD / 32;                  // 32-row tiles of O^T
+    constexpr int kKRowBytes = HD * 2;            // K tile row (one key)
+    constexpr int kKChunks = HD / 8;              // 16-byte chunks per K row
+    constexpr int kKSwzDiv = 16 / kKChunks;       // K rows per 256 bytes of LDS: rows that start in the same bank
     constexpr int kKTileBytes = kApKeys * kKRowBytes;
-    constexpr int kVRowBytes = kApKeys * 2;      // V^T tile row (one dim): 128 bytes
+    constexpr int kVRowBytes = kApKeys * 2;       // V^T tile row (one dim): 128 bytes = 8 chunks
     constexpr int kVTileBytes = HD * kVRowBytes;
-    constexpr int kKLoads = kApKeys * kKChunks / kApThreads; // 16-byte chunks per thread and tile
-    constexpr int kVLoads = HD * 8 / kApThreads;
-    __shared__ __attribute__((aligned(16))) unsigned char lds[kKTileBytes + kVTileBytes];
-    unsigned char *lds_k = lds, *lds_v = lds + kKTileBytes;
+    constexpr int kStageBytes = kKTileBytes + kVTileBytes;
+    constexpr int kKIssues = kKTileBytes / 4096;  // wavefront-wide 1 KiB loads per wavefront and tile
+    constexpr int kVIssues = kVTileBytes / 4096;
+    constexpr int kMergeFloats = 64 * (kDT * 16 + 2); // one key half's (O, m, l), a float per lane and value
+    constexpr int kOutRowHalves = HD + 8;         // padded row of the f16 output tile
+    constexpr int kOutOffset = 2 * kMergeFloats * 4;
+    static_assert(kOutOffset + 2 * 32 * kOutRowHalves * 2 <= 2 * kStageBytes, "epilogue buffers reuse the tile stages");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int qg = wave & 1, kh = wave >> 1;
     const int col = lane & 31, half = lane >> 5;
-    const int head = blockIdx.y;
-    const int qblock = blockIdx.x * kApQueries;
-    const int q0 = qblock + wave * 32;           // this wavefront's first query
     const int n = p.n;
-    const int my_q = q0 + col;                   // the query this lane's accumulator column belongs to
+    const int n_qblocks = (n + kApQueries - 1) / kApQueries;
+    // Heavy query blocks first.  When every workgroup is resident at once (two per compute unit) the second half of the
+    // grid runs upwards from the lightest block, so that workgroups b and b + grid / 2 together hold a constant number of
+    // key tiles.
+    int qi, head;
+    {
+        const int b = blockIdx.x;
+        const int rank = b / p.n_heads;           // 0 .. n_qblocks - 1 in launch order
+        head = b - rank * p.n_heads;
+        if (p.order == 0) qi = rank;
+        else if (p.order == 1) qi = n_qblocks - 1 - rank;
+        else {
+            const int top = (n_qblocks + 1) / 2;  // blocks taken from the top, descending
+            qi = rank < top ? n_qblocks - 1 - rank : rank - top;
+        }
+    }
+    const int qblock = qi * kApQueries;
+    const int q0 = qblock + qg * 32;              // this wavefront's first query
+    const int my_q = q0 + col;                    // the query this lane's accumulator column belongs to
 
     const half_t *kbase = reinterpret_cast<const half_t *>(p.cache_k) + (size_t)head * p.max_seq_len * HD;
     const half_t *vbase = reinterpret_cast<const half_t *>(p.v_t) + (size_t)head * HD * p.t_pad;
@@ -78,109 +105,92 @@ __global__ __launch_bounds__(kApThreads) void attn_prefill_kernel(AttnPrefillPar
         for (int v = 0; v < 16; v++) o_acc[d][v] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;
 
-    // keys 0 .. qblock + 127 matter to this workgroup (causal), i.e. key tiles 0 .. n_tiles - 1
-    const int last_q = min(qblock + kApQueries, n) - 1;
-    const int n_tiles = last_q / kApKeys + 1;
+    // keys 0 .. qblock + 63 matter to this workgroup (causal), i.e. key tiles 0 .. qi
+    const int n_tiles = qi + 1;
 
-    // global -> register staging of one key tile: K rows [key][hd], V^T rows [dim][key]
-    uint4_t kreg[kKLoads], vreg[kVLoads];
-    auto load_tile = [&](int kt) {
+    // ---- staging.  Load i of wavefront w fills LDS bytes (4 i + w) * 1024 .. + 1024 of the tile; lane l's 16 bytes are
+    //      chunk position l % chunks of row l / chunks, which holds the row's chunk (position ^ f(row)): consecutive
+    //      rows put the same logical chunk into different banks, which makes the MFMA operand reads conflict-free.
+    const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds;
+    int k_row[kKIssues], k_off[kKIssues], v_off[kVIssues];
 #pragma unroll
-        for (int i = 0; i < kKLoads; i++) {
-            const int c = tid + i * kApThreads;
-            const int row = c / kKChunks, ch = c % kKChunks;
-            const int key = min(kt * kApKeys + row, p.max_seq_len - 1); // keys past the sequence are masked below
-            kreg[i] = *reinterpret_cast<const uint4_t *>(kbase + (size_t)key * HD + ch * 8);
+    for (int i = 0; i < kKIssues; i++) {
+        const int L = (i * 4 + wave) * 64 + lane;
+        const int row = L / kKChunks, cp = L % kKChunks;
+        k_row[i] = row;
+        k_off[i] = (cp ^ ((row / kKSwzDiv) & (kKChunks - 1))) * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < kVIssues; i++) {
+        const int L = (i * 4 + wave) * 64 + lane;
+        const int row = L / 8, cp = L % 8;
+        v_off[i] = row * p.t_pad + (cp ^ ((row >> 1) & 7)) * 8;
+    }
+    auto issue = [&](int kt) {
+        const unsigned dst = lds_base + (unsigned)(kt & 1) * kStageBytes + (unsigned)wave * 1024;
+#pragma unroll
+        for (int i = 0; i < kKIssues; i++) {
+            const int key = min(kt * kApKeys + k_row[i], p.max_seq_len - 1); // keys past the sequence are masked below
+            dma16(kbase + (size_t)key * HD + k_off[i], dst + i * 4096);
         }
 #pragma unroll
-        for (int i = 0; i < kVLoads; i++) {
-            const int c = tid + i * kApThreads;
-            const int row = c / 8, ch = c % 8;
-            vreg[i] = *reinterpret_cast<const uint4_t *>(vbase + (size_t)row * p.t_pad + kt * kApKeys + ch * 8);
-        }
-    };
-    // LDS placement: 16-byte chunk c of row r goes to chunk c ^ f(r), so that the MFMA operand reads of consecutive
-    // rows fall into different banks
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int i = 0; i < kKLoads; i++) {
-            const int c = tid + i * kApThreads;
-            const int row = c / kKChunks, ch = c % kKChunks;
-            *reinterpret_cast<uint4_t *>(lds_k + row * kKRowBytes + ((ch ^ (row & (kKChunks - 1))) << 4)) = kreg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < kVLoads; i++) {
-            const int c = tid + i * kApThreads;
-            const int row = c / 8, ch = c % 8;
-            // rows with bit 4 set keep the two 8-byte halves of every chunk swapped: a half-wave reads one 8-byte half per
-            // row of 32 consecutive rows, and rows r and r + 16 would otherwise meet in the same banks
-            const uint4_t vv = (row & 16) ? uint4_t{vreg[i][2], vreg[i][3], vreg[i][0], vreg[i][1]} : vreg[i];
-            *reinterpret_cast<uint4_t *>(lds_v + row * kVRowBytes + ((ch ^ ((row >> 1) & 7)) << 4)) = vv;
-        }
+        for (int i = 0; i < kVIssues; i++) dma16(vbase + (size_t)(kt * kApKeys) + v_off[i], dst + kKTileBytes + i * 4096);
     };
 
-    load_tile(0);
+    const float c2 = p.scale * 1.44269504088896340736f;
+    issue(0);
     for (int kt = 0; kt < n_tiles; kt++) {
-        __syncthreads(); // everybody is done with the previous tile
-        store_tile();
-        __syncthreads();
-        if (kt + 1 < n_tiles) load_tile(kt + 1);
-        const int key0 = kt * kApKeys;
-        if (key0 > q0 + 31) continue; // every key of this tile lies after every query of this wavefront (barriers are above)
+        wait_vmcnt<0>();  // this wavefront's part of tile kt has landed
+        __syncthreads();  // ... and everybody's; everybody is done with tile kt - 1, whose stage is loaded next
+        if (kt + 1 < n_tiles) issue(kt + 1);
+        const int kg = kt * kApKeys + kh * 32; // first key of this wavefront's group
+        if (kg > q0) continue;                 // (both are multiples of 32) every key lies after every query: all masked
+        const unsigned char *lds_k = lds + (kt & 1) * kStageBytes, *lds_v = lds_k + kKTileBytes;
 
-        // ---- S^T for the two 32-key groups of the tile
-        float16_t s_acc[2];
+        // ---- S^T for the 32-key group
+        float16_t s_acc;
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
+        for (int v = 0; v < 16; v++) s_acc[v] = 0.0f;
+        {
+            const int krow = kh * 32 + col;
+            const unsigned char *rowp = lds_k + krow * kKRowBytes;
+            const int sw = (krow / kKSwzDiv) & (kKChunks - 1);
 #pragma unroll
-            for (int v = 0; v < 16; v++) s_acc[j][v] = 0.0f;
-            if (key0 + j * 32 <= q0 + 31) { // wave-uniform: otherwise the whole group is masked
-                const int krow = j * 32 + col;
-#pragma unroll
-                for (int ks = 0; ks < kKS; ks++) {
-                    const int ch = ks * 2 + half;
-                    const half8_t kf = *reinterpret_cast<const half8_t *>(lds_k + krow * kKRowBytes + ((ch ^ (krow & (kKChunks - 1))) << 4));
-                    s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, q_hi[ks], s_acc[j], 0, 0, 0);
-                    s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, q_lo[ks], s_acc[j], 0, 0, 0);
-                }
+            for (int ks = 0; ks < kKS; ks++) {
+                const half8_t kf = *reinterpret_cast<const half8_t *>(rowp + (((ks * 2 + half) ^ sw) << 4));
+                s_acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, q_hi[ks], s_acc, 0, 0, 0);
+                s_acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, q_lo[ks], s_acc, 0, 0, 0);
             }
         }
         // ---- scale (transformer.rs:768-770), causal mask (tensor.rs:496-508: col >= row + 1 is -inf), streaming softmax.
-        //      The vector ALU is what this kernel waits for, so the work per score is kept small: the maximum is taken on
-        //      the raw scores (the scale is positive), scale and log2(e) are folded into one multiplier of an exp2
-        //      (exp(scale s - scale m) = exp2(c s - c m), one fused multiply-add and one v_exp_f32 per score; the
-        //      argument error is a few 1e-6 relative in the probability), the mask is applied only on tiles that reach
-        //      the diagonal, and the accumulator is rescaled only when some row's maximum moved.
-        if (key0 + kApKeys - 1 > q0) { // some key of the tile lies after some query of this wavefront
+        //      The work per score is kept small: the maximum is taken on the raw scores (the scale is positive), scale
+        //      and log2(e) are folded into one multiplier of an exp2 (exp(scale s - scale m) = exp2(c s - c m), one fused
+        //      multiply-add and one v_exp_f32 per score; the argument error is a few 1e-6 relative in the probability),
+        //      the mask is applied only on groups that reach the diagonal, and the accumulator is rescaled only when
+        //      some row's maximum moved.
+        if (kg + 31 > q0) { // some key of the group lies after some query of this wavefront
 #pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int key = key0 + j * 32 + (v >> 2) * 8 + half * 4 + (v & 3);
-                    if (key > my_q) s_acc[j][v] = -INFINITY;
-                }
+            for (int v = 0; v < 16; v++) {
+                const int key = kg + (v >> 2) * 8 + half * 4 + (v & 3);
+                if (key > my_q) s_acc[v] = -INFINITY;
+            }
         }
         float m_tile = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) m_tile = fmaxf(m_tile, s_acc[j][v]);
+        for (int v = 0; v < 16; v++) m_tile = fmaxf(m_tile, s_acc[v]);
         m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-        // the tile holds at least key0 <= q0 <= my_q, so m_tile is finite
-        const float c2 = p.scale * 1.44269504088896340736f;
+        // the group holds key kg <= q0 <= my_q, so m_tile is finite
         const float m_new = fmaxf(m_run, m_tile);
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2); // first tile: exp2(-inf) = 0
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2); // first group: exp2(-inf) = 0
         m_run = m_new;
         const float mc = m_new * c2;
         float l_tile = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const float e = __builtin_amdgcn_exp2f(fmaf(s_acc[j][v], c2, -mc)); // masked: exp2(-inf) = 0
-                s_acc[j][v] = e;
-                l_tile += e;
-            }
+        for (int v = 0; v < 16; v++) {
+            const float e = __builtin_amdgcn_exp2f(fmaf(s_acc[v], c2, -mc)); // masked: exp2(-inf) = 0
+            s_acc[v] = e;
+            l_tile += e;
+        }
         l_run = l_run * alpha + l_tile; // this lane's half of the row; the halves are added at the end
         if (!__all(alpha == 1.0f)) {
 #pragma unroll
@@ -189,64 +199,82 @@ __global__ __launch_bounds__(kApThreads) void attn_prefill_kernel(AttnPrefillPar
                 for (int v = 0; v < 16; v++) o_acc[d][v] *= alpha;
         }
 
-        // ---- O^T += V^T . P, probabilities split hi + lo.  k slot i of lane half h in 16-slot slab s of group j is key
-        //      32 j + 16 s + 8 (i / 4) + 4 h + i % 4: the order the accumulator holds them in
+        // ---- O^T += V^T . P, probabilities split hi + lo
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            if (key0 + j * 32 > q0 + 31) continue; // all probabilities of the group are zero
+        for (int s = 0; s < 2; s++) {
+            // hi = the probability rounded towards zero, lo = the rest (exact in fp32, then rounded): hi + lo carries 22
+            // bits whichever way hi is rounded, and the packed conversion makes two halves per instruction
+            half8_t p_hi, p_lo;
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                half8_t p_hi, p_lo;
+            for (int i = 0; i < 8; i += 2) {
+                const float pa = s_acc[s * 8 + i], pb = s_acc[s * 8 + i + 1];
+                const half2_t h = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(pa, pb));
+                const half2_t l = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(pa - (float)h[0], pb - (float)h[1]));
+                p_hi[i] = h[0];
+                p_hi[i + 1] = h[1];
+                p_lo[i] = l[0];
+                p_lo[i + 1] = l[1];
+            }
+            const int ch = (kh * 2 + s) * 2 + half; // the chunk of the V^T row that holds this lane half's 8 keys
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const float pv = s_acc[j][s * 8 + i];
-                    const half_t h = (half_t)pv;
-                    p_hi[i] = h;
-                    p_lo[i] = (half_t)(pv - (float)h);
-                }
-                const int kk = j * 32 + s * 16 + half * 4; // first key (within the tile) of this lane's slots 0..3; slots 4..7: + 8
-#pragma unroll
-                for (int d = 0; d < kDT; d++) {
-                    const int vrow = d * 32 + col;
-                    const unsigned char *rowp = lds_v + vrow * kVRowBytes;
-                    const int sw = (vrow >> 1) & 7;
-                    const int sub = (((kk & 4) << 1)) ^ ((vrow & 16) >> 1); // which 8-byte half of the chunk (halves swapped in rows with bit 4 set)
-                    const half4_t a0 = *reinterpret_cast<const half4_t *>(rowp + ((((kk) >> 3) ^ sw) << 4) + sub);
-                    const half4_t a1 = *reinterpret_cast<const half4_t *>(rowp + ((((kk + 8) >> 3) ^ sw) << 4) + sub);
-                    half8_t vf;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        vf[i] = a0[i];
-                        vf[4 + i] = a1[i];
-                    }
-                    o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, p_hi, o_acc[d], 0, 0, 0);
-                    o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, p_lo, o_acc[d], 0, 0, 0);
-                }
+            for (int d = 0; d < kDT; d++) {
+                const int vrow = d * 32 + col;
+                const half8_t vf = *reinterpret_cast<const half8_t *>(lds_v + vrow * kVRowBytes + ((ch ^ ((vrow >> 1) & 7)) << 4));
+                o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, p_hi, o_acc[d], 0, 0, 0);
+                o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, p_lo, o_acc[d], 0, 0, 0);
             }
         }
     }
 
-    // ---- normalise, round to f16 (transformer.rs:793-796) and write row my_q, columns head * HD + dim of wo's input
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    if (my_q < n) {
-        half_t *orow = reinterpret_cast<half_t *>(p.out) + (size_t)my_q * p.dim + head * HD;
+    // ---- merge the two key halves: wavefront (g, 1) hands (O, m, l) to wavefront (g, 0) through LDS
+    __syncthreads(); // every wavefront is done with the tiles (all loads were waited for above)
+    float *mb = reinterpret_cast<float *>(lds) + qg * kMergeFloats + lane;
+    if (kh == 1) {
+#pragma unroll
+        for (int d = 0; d < kDT; d++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) mb[(d * 16 + v) * 64] = o_acc[d][v];
+        mb[(kDT * 16) * 64] = m_run;
+        mb[(kDT * 16 + 1) * 64] = l_run;
+    }
+    __syncthreads();
+    if (kh == 1) return;
+    {
+        const float m1 = mb[(kDT * 16) * 64], l1 = mb[(kDT * 16 + 1) * 64];
+        const float m = fmaxf(m_run, m1); // m_run is finite (key 0 <= every query); m1 is -inf if the half saw no key
+        const float a0 = __builtin_amdgcn_exp2f((m_run - m) * c2), a1 = __builtin_amdgcn_exp2f((m1 - m) * c2);
+        const float l_half = l_run * a0 + l1 * a1;
+        const float l_tot = l_half + __shfl_xor(l_half, 32, 64);
+        const float inv0 = a0 / l_tot, inv1 = a1 / l_tot;
+        // normalise, round to f16 (transformer.rs:793-796) and turn O^T into rows of the output through LDS, so that
+        // the stores to memory are whole 16-byte pieces of consecutive columns
+        half_t *ot = reinterpret_cast<half_t *>(lds + kOutOffset) + qg * (32 * kOutRowHalves);
 #pragma unroll
         for (int d = 0; d < kDT; d++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 half4_t o;
 #pragma unroll
-                for (int i = 0; i < 4; i++) o[i] = (half_t)(o_acc[d][g * 4 + i] / l_tot);
-                *reinterpret_cast<half4_t *>(orow + d * 32 + g * 8 + half * 4) = o;
+                for (int i = 0; i < 4; i++) o[i] = (half_t)(o_acc[d][g * 4 + i] * inv0 + mb[(d * 16 + g * 4 + i) * 64] * inv1);
+                *reinterpret_cast<half4_t *>(ot + col * kOutRowHalves + d * 32 + g * 8 + half * 4) = o;
             }
+        // rows q0 .. q0 + 31, columns head * HD .. + HD of wo's input
+        half_t *obase = reinterpret_cast<half_t *>(p.out) + (size_t)head * HD;
+#pragma unroll
+        for (int i = 0; i < 32 * kKChunks / 64; i++) {
+            const int c = i * 64 + lane;
+            const int r = c / kKChunks, ch = c % kKChunks;
+            if (q0 + r < n)
+                *reinterpret_cast<half8_t *>(obase + (size_t)(q0 + r) * p.dim + ch * 8) = *reinterpret_cast<const half8_t *>(ot + r * kOutRowHalves + ch * 8);
+        }
     }
 }
 
 bool attn_prefill_supported(int head_dim) { return head_dim == 64 || head_dim == 128; }
 
 hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s) {
-    if (p.n < 1 || p.n_heads < 1 || (p.t_pad % kApKeys) != 0 || p.t_pad < p.n || (p.dim % 4) != 0) return hipErrorInvalidValue;
-    dim3 grid((p.n + kApQueries - 1) / kApQueries, p.n_heads);
+    if (p.n < 1 || p.n_heads < 1 || (p.t_pad % kApKeys) != 0 || p.t_pad < p.n || (p.dim % 8) != 0 || p.max_seq_len < 1) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)((p.n + kApQueries - 1) / kApQueries * p.n_heads));
     switch (p.head_dim) {
     case 64: hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, dim3(kApThreads), 0, s, p); break;
     case 128: hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, dim3(kApThreads), 0, s, p); break;

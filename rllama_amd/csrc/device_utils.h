@@ -107,4 +107,18 @@ __device__ __forceinline__ void rope_pair(float re, float im, float2 f, float &o
     oim = p2 + p3;
 }
 
+// One direct-to-LDS load: lane l's 16 bytes at `src` land at LDS byte address dst + 16 l (dst is wave-uniform and
+// travels in M0).  Written as inline assembly on purpose: through the builtin the compiler tracks the load as an LDS
+// write and puts s_waitcnt vmcnt(0) in front of every LDS read, which would also wait for the prefetched K-tiles;
+// here the waits are placed by hand (vmcnt is decremented in issue order).
+__device__ __forceinline__ void dma16(const half_t *src, unsigned dst) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory");
+}
+
+template <int kN>
+__device__ __forceinline__ void wait_vmcnt() { // s_waitcnt vmcnt(kN) only (6-bit count: bits 3:0 and 15:14)
+    static_assert(kN >= 0 && kN < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kN & 0xF) | ((kN >> 4) << 14));
+}
+
 } // namespace rlh

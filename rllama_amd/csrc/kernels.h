@@ -111,15 +111,17 @@ struct PrefillRopeParams {
     void *v_t;              // [n_heads][head_dim][t_pad] f16
     int n, dim, head_dim, max_seq_len, t_pad;
     int q_stride;
+    int vt_swap;            // 1: positions within v_t rows have bits 2 and 3 swapped (the order attn_prefill_kernel reads)
 };
 // fused causal attention of a multi-token forward (attn_prefill.hip); head_dim 64 or 128, f16 cache
 struct AttnPrefillParams {
     const void *q2;          // [n_heads][n] rows [q hi (head_dim) | q lo (head_dim)] f16, after RoPE
     const void *cache_k;     // this layer: [n_heads][max_seq_len][head_dim] f16
-    const void *v_t;         // [n_heads][head_dim][t_pad] f16 (V transposed, finite values in the padding)
+    const void *v_t;         // [n_heads][head_dim][t_pad] f16 (V transposed with vt_swap, finite values in the padding)
     void *out;               // [n][dim] f16: head h at columns h * head_dim ..
     int n, n_heads, head_dim, dim, max_seq_len, t_pad;
     float scale;             // 1 / sqrt(head_dim) (transformer.rs:770)
+    int order;               // launch order of the query blocks: 0 ascending, 1 descending, 2 descending then ascending
 };
 bool attn_prefill_supported(int head_dim);
 hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s);

@@ -142,6 +142,8 @@ __global__ __launch_bounds__(256) void rope_kv_prefill_tiled_kernel(PrefillRopeP
         const int rr = c / chunks, ch = c - rr * chunks;
         const int r = r0 + rr;
         const int j = head * hd + ch * 8; // first of this piece's 8 dims within the row of q / k / v
+        // position of this row in the transposed V tile
+        const int rs = p.vt_swap ? (rr & ~12) | ((rr & 4) << 1) | ((rr & 8) >> 1) : rr;
         h8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
         if (r < p.n) {
             const half_t *row = qkv + (size_t)r * 3 * p.dim;
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(256) void rope_kv_prefill_tiled_kernel(PrefillRopeP
             *reinterpret_cast<h8 *>(cv + co) = v8;
         }
 #pragma unroll
-        for (int e = 0; e < 8; e++) vt_tile[(ch * 8 + e) * kPad + rr] = v8[e]; // zeros for positions past n: finite padding
+        for (int e = 0; e < 8; e++) vt_tile[(ch * 8 + e) * kPad + rs] = v8[e]; // zeros for positions past n: finite padding
     }
     __syncthreads();
     half_t *vt = reinterpret_cast<half_t *>(p.v_t) + (size_t)head * hd * p.t_pad + r0;
@@ -188,6 +190,7 @@ hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s) {
         hipLaunchKernelGGL(rope_kv_prefill_tiled_kernel, dim3((p.n + kRopeTileRows - 1) / kRopeTileRows, n_heads), dim3(256), 0, s, p);
         return hipGetLastError();
     }
+    if (p.vt_swap) return hipErrorInvalidValue; // only the tiled kernel writes the swapped order
     const size_t total = (size_t)p.n * (p.dim / 2);
     const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
     hipLaunchKernelGGL(rope_kv_prefill_kernel, dim3(blocks), dim3(256), 0, s, p);
