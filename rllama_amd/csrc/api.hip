@@ -792,6 +792,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     S.release();
     const size_t d = (size_t)m->prm.dim, F = (size_t)m->prm.ffn_hidden, H = (size_t)m->prm.n_heads, hd = (size_t)m->head_dim;
     const size_t N = (size_t)n, tp = (N + 63) & ~(size_t)63;
+    const size_t es = m->prm.force_f16 ? 2 : 4; // element size of the activations between the GEMMs
     hipError_t e = hipSuccess;
     auto A = [&](void **p, size_t bytes) {
         if (e != hipSuccess) return;
@@ -800,16 +801,16 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     };
     A((void **)&S.x, N * d * 4);
     A((void **)&S.h, N * d * 4);
-    A((void **)&S.xn, N * d * 2);
-    A((void **)&S.qkv, N * 3 * d * 2);
-    A((void **)&S.q2, N * d * 2 * 2);
-    A((void **)&S.v_t, H * hd * tp * 2);
+    A((void **)&S.xn, N * d * es);
+    A((void **)&S.qkv, N * 3 * d * es);
+    A((void **)&S.q2, N * d * 2 * 2); // f16 mode: hi and lo halves; f32 mode: one float
+    A((void **)&S.v_t, H * hd * tp * es);
     A((void **)&S.scores, H * N * tp * 4);
-    A((void **)&S.p2, H * N * tp * 2 * 2);
-    A((void **)&S.a, N * d * 2);
-    A((void **)&S.g, N * F * 2);
-    A((void **)&S.u, N * F * 2);
-    A((void **)&S.mm, N * F * 2);
+    if (es == 2) A((void **)&S.p2, H * N * tp * 2 * 2); // f32 mode turns the scores into probabilities in place
+    A((void **)&S.a, N * d * es);
+    A((void **)&S.g, N * F * es);
+    A((void **)&S.u, N * F * es);
+    A((void **)&S.mm, N * F * es);
     if (e == hipSuccess) e = hipStreamSynchronize(m->ctx->stream);
     if (e != hipSuccess) {
         S.release();
@@ -960,6 +961,125 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     return RLH_OK;
 }
 
+// f32 mode can take the matrix-core path when every K extent is a whole number of 32-float K-tiles
+static bool prefill_f32_supported(const rlh_model *m) {
+    return m->prm.dim % 32 == 0 && m->prm.ffn_hidden % 32 == 0 && m->head_dim % 32 == 0;
+}
+
+// Multi-token forward at start_pos == 0 in f32 mode: the same structure as enqueue_prefill on fp32 operands
+// (v_mfma_f32_32x32x2_f32), no rounding points, residual adds as accumulating GEMM epilogues on x in place.
+static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n) {
+    int rc = ensure_prefill_scratch(m, n);
+    if (rc != RLH_OK) return rc;
+    hipStream_t st = m->ctx->stream;
+    const rlh_model_params &P = m->prm;
+    PrefillScratch &S = m->pf;
+    const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size, H = P.n_heads, hd = m->head_dim;
+    const int tp = (n + 63) & ~63;
+    const float eps = (float)P.norm_eps;
+    HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
+    HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));
+    HIP_TRY(launch_embed_rows(m->tok_emb.p, m->tok_emb.f16, m->prompt_dev, n, d, S.x, st));
+    const size_t layer_elems = (size_t)H * P.max_seq_len * hd;
+    auto gemm = [&](const void *a, int lda, const void *b, int ldb, float *cc, int ldc, int mm, int nn, int kk, int accumulate) -> int {
+        GemmParams g{};
+        g.a = (const _Float16 *)a;
+        g.b = (const _Float16 *)b;
+        g.c = cc;
+        g.m = mm;
+        g.n = nn;
+        g.k = kk;
+        g.lda = lda;
+        g.ldb = ldb;
+        g.ldc = ldc;
+        g.batch = 1;
+        g.accumulate = accumulate;
+        g.f32_operands = 1;
+        HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
+        return RLH_OK;
+    };
+    float *xn = (float *)S.xn, *qkv = (float *)S.qkv, *q = (float *)S.q2, *v_t = (float *)S.v_t, *att = (float *)S.a;
+    float *gg = (float *)S.g, *uu = (float *)S.u, *mm = (float *)S.mm;
+    for (int l = 0; l < P.n_layers; l++) {
+        Layer &L = m->layers[(size_t)l];
+        float *ck = (float *)c->k + (size_t)l * layer_elems;
+        float *cv = (float *)c->v + (size_t)l * layer_elems;
+        HIP_TRY(launch_rmsnorm_rows_f32(xn, S.x, (const float *)L.attn_norm.p, n, d, eps, st));
+        if ((rc = gemm(xn, d, L.wqkv.p, d, qkv, 3 * d, n, 3 * d, d, 0)) != RLH_OK) return rc;
+        PrefillRopeF32Params rp{};
+        rp.qkv = qkv;
+        rp.freqs = m->freqs;
+        rp.q = q;
+        rp.cache_k = ck;
+        rp.cache_v = cv;
+        rp.v_t = v_t;
+        rp.n = n;
+        rp.dim = d;
+        rp.head_dim = hd;
+        rp.max_seq_len = P.max_seq_len;
+        rp.t_pad = tp;
+        HIP_TRY(launch_rope_kv_prefill_f32(rp, st));
+        {   // scores[h] = q[h] . K[h]^T, tiles above the diagonal skipped (transformer.rs:762-770)
+            GemmParams g{};
+            g.a = (const _Float16 *)q;
+            g.b = (const _Float16 *)ck;
+            g.c = S.scores;
+            g.m = n;
+            g.n = n;
+            g.k = hd;
+            g.causal = 1;
+            g.lda = hd;
+            g.ldb = hd;
+            g.ldc = tp;
+            g.batch = H;
+            g.stride_a = (size_t)n * hd;
+            g.stride_b = (size_t)P.max_seq_len * hd;
+            g.stride_c = (size_t)n * tp;
+            g.f32_operands = 1;
+            HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
+        }
+        HIP_TRY(launch_causal_softmax_f32(S.scores, H, n, tp, hd, st));
+        {   // out[h] = P[h] . V[h], written as columns h * hd .. of the [n x dim] input of wo (transformer.rs:777-796)
+            GemmParams g{};
+            g.a = (const _Float16 *)S.scores;
+            g.b = (const _Float16 *)v_t;
+            g.c = att;
+            g.m = n;
+            g.n = hd;
+            g.k = tp;
+            g.causal = 2;
+            g.lda = tp;
+            g.ldb = tp;
+            g.ldc = d;
+            g.batch = H;
+            g.stride_a = (size_t)n * tp;
+            g.stride_b = (size_t)hd * tp;
+            g.stride_c = (size_t)hd;
+            g.f32_operands = 1;
+            HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
+        }
+        if ((rc = gemm(att, d, L.wo.p, d, S.x, d, n, d, d, 1)) != RLH_OK) return rc;     // x += wo(att)   (transformer.rs:442)
+        HIP_TRY(launch_rmsnorm_rows_f32(xn, S.x, (const float *)L.ffn_norm.p, n, d, eps, st));
+        if ((rc = gemm(xn, d, L.w1.p, d, gg, F, n, F, d, 0)) != RLH_OK) return rc;
+        if ((rc = gemm(xn, d, L.w3.p, d, uu, F, n, F, d, 0)) != RLH_OK) return rc;
+        HIP_TRY(launch_silu_mul_f32(gg, uu, mm, (size_t)n * F, st));
+        if ((rc = gemm(mm, F, L.w2.p, F, S.x, d, n, d, F, 1)) != RLH_OK) return rc;      // x += w2(...)   (transformer.rs:445)
+    }
+    // final norm + output head on the last row only (transformer.rs:378-381)
+    GemvParams p{};
+    p.stream_weights = m->stream_weights;
+    p.w = m->output.p;
+    p.w_is_f16 = m->output.f16;
+    p.x = S.x + (size_t)(n - 1) * d;
+    p.norm_w = (const float *)m->norm.p;
+    p.eps = eps;
+    p.y = m->logits;
+    p.n_rows = V;
+    p.k = d;
+    HIP_TRY(launch_gemv(p, kEpiStore, st));
+    return RLH_OK;
+}
+
 static int check_forward_args(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, const char *who) {
     if (!m || !c || !tokens) return fail(RLH_ERR_INVALID, "%s: NULL argument", who);
     if (c->model != m) return fail(RLH_ERR_STATE, "%s: caches belong to another model", who);
@@ -982,7 +1102,10 @@ static int enqueue_forward(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     hipStream_t st = m->ctx->stream;
     m->next_pos = -1;
     m->greedy_caches = nullptr;
-    if (n > 1 && m->prm.force_f16 && m->prefill_mode == 0) return enqueue_prefill(m, c, tokens, n);
+    if (n > 1 && m->prefill_mode == 0) {
+        if (m->prm.force_f16) return enqueue_prefill(m, c, tokens, n);
+        if (prefill_f32_supported(m)) return enqueue_prefill_f32(m, c, tokens, n);
+    }
     HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
     HIP_TRY(launch_set_state(m->state, start_pos, tokens[0], 1, st));
     for (int i = 0; i < n; i++) {
@@ -1398,8 +1521,8 @@ extern "C" int rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tens
     CtxLock lock(dst->ctx);
     hipStream_t st = dst->ctx->stream;
     const int n = src->rows, k = src->cols, mrows = other->rows;
-    if (f16 && n > 1) {
-        // more than one row of f16: the matrix-core GEMM (f32 operands keep the per-row path below)
+    if (n > 1 && (f16 || k % 32 == 0)) {
+        // more than one row: the matrix-core GEMM (fp32 operands need whole K-tiles of 32, else the per-row path below)
         GemmParams g{};
         g.a = (const _Float16 *)src->p;
         g.b = (const _Float16 *)other->p;
@@ -1411,7 +1534,8 @@ extern "C" int rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tens
         g.ldb = k;
         g.ldc = mrows;
         g.batch = 1;
-        HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
+        g.f32_operands = f16 ? 0 : 1;
+        HIP_TRY(launch_gemm_f16(g, f16 ? kGemmEpiF16 : kGemmEpiF32, st));
         return RLH_OK;
     }
     float *xf = nullptr, *yf = nullptr;

@@ -127,6 +127,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_f16_kernel(GemmParams p) {
 }
 
 hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s) {
+    if (p.f32_operands) { // fp32 operands exist on the fast path only
+        if (p.m <= 0 || p.n <= 0 || p.batch < 1 || !gemm_f16_dma_supported(p)) return hipErrorInvalidValue;
+        return launch_gemm_f16_dma(p, epilogue, s);
+    }
     if (p.m <= 0 || p.n <= 0 || p.k <= 0 || (p.k % 8) != 0 || (p.lda % 8) != 0 || (p.ldb % 8) != 0 || p.batch < 1) return hipErrorInvalidValue;
     // RLLAMA_HIP_GEMM_SIMPLE=1 keeps every product on the kernel of this file (tuning / cross-checks)
     static const bool simple_only = getenv("RLLAMA_HIP_GEMM_SIMPLE") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_SIMPLE")) != 0;

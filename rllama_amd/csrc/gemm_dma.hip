@@ -26,8 +26,12 @@ typedef __attribute__((ext_vector_type(16))) float float16_t;
 
 // kWavesM: wavefront rows (tile height 64 kWavesM); kNT: 32-column MFMA tiles per wavefront (tile width 64 kNT);
 // kBK: halves of K per tile (32 or 64); kStages: LDS stages (K-tiles in flight).
-template <int kEpi, int kWavesM, int kNT, int kBK, int kStages>
+// kF32: the operands are fp32 (f32 mode: tensor.rs:1282-1475 for src.rows > 1).  Staging moves bytes and is the same
+// with a row of kBK / 2 floats; a 16-byte fragment then holds 4 consecutive k of a row and feeds 4
+// v_mfma_f32_32x32x2_f32 (k slot of lane half h in the j-th of them: float j of chunk 2 ks + h, for A and B alike).
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false>
 __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams p) {
+    constexpr int kE = kF32 ? 2 : 1;                     // halves per operand element: k, lda, ldb, strides count elements
     constexpr int kWaves = 2 * kWavesM;
     constexpr int kBM = 64 * kWavesM, kBN = 64 * kNT;
     constexpr int kCpr = kBK / 8;                        // 16-byte chunks per LDS row
@@ -46,13 +50,13 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     const int wm = wave >> 1, wn = wave & 1;
     const int bm0 = blockIdx.y * kBM, bn0 = blockIdx.x * kBN;
     const size_t zb = blockIdx.z;
-    const half_t *A = p.a + zb * p.stride_a;
-    const half_t *B = p.b + zb * p.stride_b;
-    const int M = p.m, N = p.n, K = p.k;
+    const half_t *A = p.a + zb * p.stride_a * kE;
+    const half_t *B = p.b + zb * p.stride_b * kE;
+    const int M = p.m, N = p.n, K = p.k * kE;          // K, segments and k offsets below are in halves
     if (p.causal == 1 && bn0 > bm0 + kBM - 1) return; // the whole tile lies above the diagonal (uniform for the workgroup)
     // K-tiles: n_seg segments of tps tiles each; A's k runs on from segment to segment, B's starts over
-    const int seg_len = p.k_seg > 0 ? p.k_seg : K;
-    const int seg_used = p.causal == 2 ? min(seg_len, (bm0 + kBM + kBK - 1) / kBK * kBK) : seg_len;
+    const int seg_len = p.k_seg > 0 ? p.k_seg * kE : K;
+    const int seg_used = p.causal == 2 ? min(seg_len, ((bm0 + kBM) * kE + kBK - 1) / kBK * kBK) : seg_len;
     const int tps = seg_used / kBK;
     const int n_kt = (K / seg_len) * tps;
 
@@ -71,7 +75,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         const int lc = l_pc ^ ((row / kSwzDiv) % kCpr);  // logical chunk this lane fetches
         // rows past the matrix edge are clamped to a valid row; what they produce is never stored
         const int grow = is_b ? min(bn0 + row, N - 1) : min(bm0 + row, M - 1);
-        gsrc[i] = (is_b ? B + (size_t)grow * p.ldb : A + (size_t)grow * p.lda) + lc * 8;
+        gsrc[i] = (is_b ? B + (size_t)grow * p.ldb * kE : A + (size_t)grow * p.lda * kE) + lc * 8;
         src_is_b[i] = is_b;
     }
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_raw;
@@ -144,6 +148,15 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     constexpr int kKS = kBK / 16;
     static_assert(kKS % 2 == 0, "fragment sets alternate by K-step parity");
     half8_t af[2][2], bf[2][kNT];
+    auto mma = [&](const half8_t &a, const half8_t &b, float16_t &c) {
+        if constexpr (kF32) {
+            const float4_t a4 = __builtin_bit_cast(float4_t, a), b4 = __builtin_bit_cast(float4_t, b);
+#pragma unroll
+            for (int e = 0; e < 4; e++) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[e], b4[e], c, 0, 0, 0);
+        } else {
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+        }
+    };
     auto read_frags = [&](int set, const unsigned char *stage, int ks) {
         const int lc = ks * 2 + fch;
 #pragma unroll
@@ -167,12 +180,12 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
                 for (int j = 0; j < kNT; j++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+                    for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
             } else {
 #pragma unroll
                 for (int j = 0; j < kNT / 2; j++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+                    for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
                 __builtin_amdgcn_sched_barrier(0);
                 if (short_wave) wait_vmcnt<(kStages - 2) * kLoadsMin>();
                 else wait_vmcnt<(kStages - 2) * kLoadsMax>();
@@ -183,7 +196,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
                 for (int j = kNT / 2; j < kNT; j++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+                    for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
             }
         }
     }
@@ -237,22 +250,36 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 }
 
 bool gemm_f16_dma_supported(const GemmParams &p) {
-    if (p.k < kDmaMinBK || (p.k % kDmaMinBK) != 0 || (p.lda % 8) != 0 || (p.ldb % 8) != 0) return false;
-    if (p.k_seg < 0 || (p.k_seg > 0 && ((p.k % p.k_seg) != 0 || (p.k_seg % 64) != 0))) return false;
+    const int e = p.f32_operands ? 2 : 1; // halves per element
+    if (p.k * e < kDmaMinBK || ((p.k * e) % kDmaMinBK) != 0 || ((p.lda * e) % 8) != 0 || ((p.ldb * e) % 8) != 0) return false;
+    if (((p.stride_a * e) % 8) != 0 || ((p.stride_b * e) % 8) != 0) return false;
+    if (p.k_seg < 0 || (p.k_seg > 0 && ((p.k % p.k_seg) != 0 || ((p.k_seg * e) % 64) != 0))) return false;
     return p.causal >= 0 && p.causal <= 2;
 }
 
-template <int kEpi, int kWavesM, int kNT, int kBK, int kStages>
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false>
 static hipError_t launch_dma(const GemmParams &p, hipStream_t s) {
     constexpr int bm = 64 * kWavesM, bn = 64 * kNT;
     constexpr size_t lds = (size_t)kStages * (bm + bn) * kBK * 2;
     static_assert(lds <= 160 * 1024, "LDS of one compute unit");
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages>),
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) return attr;
     dim3 grid((p.n + bn - 1) / bn, (p.m + bm - 1) / bm, p.batch);
-    hipLaunchKernelGGL((gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages>), grid, dim3(128 * kWavesM), lds, s, p);
+    hipLaunchKernelGGL((gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32>), grid, dim3(128 * kWavesM), lds, s, p);
     return hipGetLastError();
+}
+
+// fp32 operands (always K-tiles of 32 floats, fp32 store / accumulate epilogue)
+static hipError_t launch_dma_f32(const GemmParams &p, int tile, hipStream_t s) {
+    switch (tile) {
+    case 0: return launch_dma<kGemmEpiF32, 2, 2, 64, 2, true>(p, s);
+    case 4: return launch_dma<kGemmEpiF32, 2, 2, 64, 4, true>(p, s);
+    case 1: return launch_dma<kGemmEpiF32, 4, 2, 64, 3, true>(p, s);
+    case 2: return launch_dma<kGemmEpiF32, 4, 3, 64, 2, true>(p, s);
+    case 3: return launch_dma<kGemmEpiF32, 4, 4, 64, 2, true>(p, s);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 template <int kEpi>
@@ -284,14 +311,15 @@ static int device_compute_units() {
 static int choose_tile(const GemmParams &p) {
     static const int forced = getenv("RLLAMA_HIP_GEMM_TILE") ? atoi(getenv("RLLAMA_HIP_GEMM_TILE")) : -1;
     if (forced >= 1 && forced <= 3) return forced;
-    if (forced == 0 && p.k % 64 == 0) return 0;
+    const int k_halves = p.k * (p.f32_operands ? 2 : 1);
+    if (forced == 0 && k_halves % 64 == 0) return 0;
     const int n_cu = device_compute_units();
     const int bms[4] = {128, 256, 256, 256}, bns[4] = {128, 128, 192, 256};
     const double eff[4] = {1.0, 0.92, 1.23, 1.15}; // relative throughput of a busy compute unit, measured on 7B shapes
     int best = -1;
     double best_t = 0.0;
     for (int t = 0; t < 4; t++) {
-        if (t == 0 && p.k % 64 != 0) continue;
+        if (t == 0 && k_halves % 64 != 0) continue;
         const long blocks = (long)((p.n + bns[t] - 1) / bns[t]) * ((p.m + bms[t] - 1) / bms[t]) * p.batch;
         const long rounds = (blocks + n_cu - 1) / n_cu;
         const double time = (double)rounds * bms[t] * bns[t] / eff[t];
@@ -308,6 +336,10 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s)
         // pipeline instead (measured on the wo / w2 products of a 1024-token 7B prefill: 108 -> 85 us per launch).
         const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128) * p.batch;
         if (blocks <= device_compute_units()) tile = 4;
+    }
+    if (p.f32_operands) {
+        if (epilogue != kGemmEpiF32 || ((p.k * 2) % 64) != 0 || (p.k_seg != 0 && ((p.k_seg * 2) % 64) != 0)) return hipErrorInvalidValue;
+        return launch_dma_f32(p, tile, s);
     }
     switch (epilogue) {
     case kGemmEpiF16: return launch_dma_epi<kGemmEpiF16>(p, tile, s);

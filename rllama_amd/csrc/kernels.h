@@ -94,6 +94,8 @@ struct GemmParams {
     int causal;             // 1: C tiles that lie entirely above the diagonal (col > row) are skipped, not written
                             // 2: of every segment only k < (last row of the C tile) + 1, rounded up to the K-tile, is used
                             //    (A holds zeros beyond the diagonal: causal probabilities times V)
+    int f32_operands;       // 1: a and b point to fp32 data (f32 mode); m, n, k, lda, ldb, strides and k_seg count elements
+                            //    all the same.  Needs k % 32 == 0 and the kGemmEpiF32 epilogue.
 };
 
 hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s);
@@ -125,6 +127,21 @@ struct AttnPrefillParams {
 };
 bool attn_prefill_supported(int head_dim);
 hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s);
+
+// f32 mode (prefill_f32.hip): the same steps on fp32 tensors, no rounding points
+struct PrefillRopeF32Params {
+    const float *qkv;       // [n x 3 dim]
+    const float2 *freqs;    // [max_seq_len x head_dim/2]
+    float *q;               // [n_heads][n][head_dim], after RoPE
+    float *cache_k, *cache_v; // this layer: [n_heads][max_seq_len][head_dim]
+    float *v_t;             // [n_heads][head_dim][t_pad]
+    int n, dim, head_dim, max_seq_len, t_pad;
+};
+hipError_t launch_rmsnorm_rows_f32(float *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s);
+hipError_t launch_rope_kv_prefill_f32(const PrefillRopeF32Params &p, hipStream_t s);
+// scores [n_heads][n] rows of t_pad floats (raw q.k) -> causal probabilities in place
+hipError_t launch_causal_softmax_f32(float *scores, int n_heads, int n, int t_pad, int head_dim, hipStream_t s);
+hipError_t launch_silu_mul_f32(const float *g, const float *u, float *m, size_t total, hipStream_t s);
 
 hipError_t launch_embed_rows(const void *table, int table_f16, const int32_t *tokens_dev, int n, int dim, float *x, hipStream_t s);
 hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s);

@@ -189,10 +189,12 @@ def test_forward_f16_mode(ctx, shape):
     gm.free()
 
 
-@pytest.mark.parametrize("n_heads,n", [(2, 300), (2, 129), (4, 64), (4, 1)], ids=["hd128-n300", "hd128-n129", "hd64-n64", "hd64-n1"])
-def test_prefill_fused_attention_head_dims(ctx, n_heads, n):
-    """The one-kernel causal attention of the multi-token forward (head_dim 128 and 64; ragged query and key tiles) against the oracle."""
-    shape = Shape(dim=256, n_layers=2, n_heads=n_heads, ffn_hidden=512, vocab_size=128, max_seq_len=320)
+@pytest.mark.parametrize("n_heads,n,cap", [(2, 300, 320), (2, 129, 320), (4, 64, 320), (4, 1, 320), (2, 289, 290), (4, 33, 35)],
+                         ids=["hd128-n300", "hd128-n129", "hd64-n64", "hd64-n1", "hd128-n289-cap290", "hd64-n33-cap35"])
+def test_prefill_fused_attention_head_dims(ctx, n_heads, n, cap):
+    """The one-kernel causal attention of the multi-token forward (head_dim 128 and 64; ragged query and key tiles, also a
+    cache whose capacity ends inside the last key tile) against the oracle."""
+    shape = Shape(dim=256, n_layers=2, n_heads=n_heads, ffn_hidden=512, vocab_size=128, max_seq_len=cap)
     W = synth_weights(shape, seed=45, std=0.08, norm_ones=False)
     toks = np.random.default_rng(46).integers(0, shape.vocab_size, n + 1)
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
@@ -388,6 +390,53 @@ def test_mfma_gemm_f16(ctx, n, m_rows, k):
     mag = np.abs(oracle.f16_bits_to_f32(a).astype(np.float64)) @ np.abs(oracle.f16_bits_to_f32(b).astype(np.float64)).T
     close_f16(got, want, mag, f"mfma gemm {n}x{m_rows}x{k}")
     assert np.mean(got != want) < 0.03
+
+
+@pytest.mark.parametrize("n,m_rows,k", [(2, 40, 32), (130, 200, 96), (300, 129, 512), (1024, 384, 256)])
+def test_mfma_gemm_f32(ctx, n, m_rows, k):
+    """fp32 src [n x k] . other[m x k]^T with n > 1 and k a multiple of 32 runs on the matrix cores (fp32 products, fp32
+    accumulation: only the order of the additions differs from tensor.rs:1282-1475); every element against a float64
+    product, with the tolerance the reference's own test uses (1e-5 scaled, tensor.rs:2554-2650), tiles straddling the edges."""
+    rng = np.random.default_rng(n * 11 + m_rows * 5 + k)
+    a = rng.uniform(-1, 1, (n, k)).astype(f32)
+    b = (rng.standard_normal((m_rows, k)) * 0.5).astype(f32)
+    got = Tensor.from_numpy(ctx, a).matrix_mul_transposed(Tensor.from_numpy(ctx, b)).to_numpy()
+    want64 = a.astype(np.float64) @ b.astype(np.float64).T
+    mag = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T
+    assert got.shape == (n, m_rows)
+    assert np.all(np.abs(got - want64) <= 3e-6 * mag + 1e-30), float(np.max(np.abs(got - want64) / mag))
+    if n * m_rows * k <= 130 * 200 * 96:   # and the oracle's own lane-ordered sum on the sizes it finishes quickly
+        assert np.allclose(got, oracle.matmul_transposed_f32(a, b), rtol=0, atol=1e-5 * k ** 0.5)
+
+
+def test_prefill_f32_mode_matrix_core_path(ctx):
+    """n > 1 at start_pos 0 in f32 mode (fp32 weights, activations and cache): the fp32 matrix-core prefill against the
+    token-by-token path and the oracle's prefill, logits and KV cache; ragged n, several row tiles, decode continues."""
+    shape = Shape(dim=256, n_layers=3, n_heads=4, ffn_hidden=704, vocab_size=512, max_seq_len=330)
+    W = random_f32_weights(shape, seed=51, std=0.08)
+    toks = np.random.default_rng(52).integers(0, shape.vocab_size, 321)
+    om, gm = make_oracle(shape, W, False), make_gpu(ctx, shape, W, False)
+    for n in (2, 33, 150, 320):
+        oc = om.make_caches()
+        want = om.forward(toks[:n], 0, oc)
+        ga, gb = gm.make_caches(), gm.make_caches()
+        gm.set_prefill_mode(False)
+        a = gm.forward(toks[:n], 0, ga)
+        gm.set_prefill_mode(True)
+        b = gm.forward(toks[:n], 0, gb)
+        gm.set_prefill_mode(False)
+        assert max_rel_err(a, want) < TOL_F32 and max_rel_err(b, want) < TOL_F32, (n, max_rel_err(a, want), max_rel_err(b, want))
+        for l in (0, shape.n_layers - 1):
+            for which in (0, 1):
+                ca, cb, co = ga.read(l, 1, which), gb.read(l, 1, which), oc.read(l, 1, which)
+                assert not np.any(ca[:, n:])
+                assert np.allclose(ca[:, :n], co[:, :n], rtol=1e-4, atol=1e-5)
+                assert np.allclose(cb[:, :n], co[:, :n], rtol=1e-4, atol=1e-5)
+        nxt = [int(toks[n])]
+        want1 = om.forward(nxt, n, oc)
+        assert max_rel_err(gm.forward(nxt, n, ga), want1) < TOL_F32
+        assert max_rel_err(gm.forward(nxt, n, gb), want1) < TOL_F32
+    gm.free()
 
 
 def test_prefill_matrix_core_path_against_token_by_token_and_oracle(ctx):
