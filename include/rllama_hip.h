@@ -111,8 +111,9 @@ int  rlh_model_get_tensor(rlh_model *model, int kind, int layer, void *host_out,
 int  rlh_model_fill_synthetic(rlh_model *model, uint64_t seed, double std);
 /* How a multi-token forward (n > 1 at start_pos == 0, src/transformer.rs:343-383) is executed.  0 (default): every
  * projection as one matrix-core GEMM over all n rows and attention as batched GEMMs around a causal softmax
- * (f16 mode; f32 mode has no f16 operands for the matrix cores and always uses mode 1).  1: token by token with
- * the decode kernels.  Both give the reference's result up to the order of fp32 additions. */
+ * (f16 mode: f16 matrix cores with the reference's rounding points; f32 mode: fp32 matrix cores, no rounding points,
+ * when dim, ffn_hidden and head_dim are multiples of 32, else mode 1).  1: token by token with the decode kernels.
+ * Both give the reference's result up to the order of fp32 additions. */
 int  rlh_model_set_prefill_mode(rlh_model *model, int mode);
 /* The layer split rule of src/transformer.rs:262-279: last_layer_on_gpu = round(p * (n_layers - 1)).
  * Reports it; all layers run on the device regardless (nothing is left on the host). */
