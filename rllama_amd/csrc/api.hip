@@ -16,6 +16,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <map>
 #include <string>
 #include <thread>
 #include <vector>
@@ -133,6 +134,8 @@ struct rlh_caches {
     void *k = nullptr, *v = nullptr;
     size_t bytes_each = 0;
     int f16 = 0;
+    // one captured decode step (token step + greedy pick) per attention grid shape, replayed by the greedy loops
+    std::map<int, hipGraphExec_t> step_graphs;
 };
 
 struct rlh_tensor {
@@ -606,6 +609,7 @@ extern "C" void rlh_caches_free(rlh_caches *c) {
     if (!c) return;
     CtxLock lock(c->ctx);
     (void)hipStreamSynchronize(c->ctx->stream);
+    for (auto &kv : c->step_graphs) (void)hipGraphExecDestroy(kv.second);
     if (c->k) (void)hipFree(c->k);
     if (c->v) (void)hipFree(c->v);
     delete c;
@@ -805,8 +809,11 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     A((void **)&S.qkv, N * 3 * d * es);
     A((void **)&S.q2, N * d * 2 * 2); // f16 mode: hi and lo halves; f32 mode: one float
     A((void **)&S.v_t, H * hd * tp * es);
-    A((void **)&S.scores, H * N * tp * 4);
-    if (es == 2) A((void **)&S.p2, H * N * tp * 2 * 2); // f32 mode turns the scores into probabilities in place
+    // the [n x n] score / probability matrices exist only in the GEMM form of attention (the one-kernel form keeps them
+    // on chip); f32 mode turns the scores into probabilities in place
+    const bool gemm_attention = !(es == 2 && m->prefill_attn_fused && attn_prefill_supported((int)hd));
+    if (gemm_attention) A((void **)&S.scores, H * N * tp * 4);
+    if (gemm_attention && es == 2) A((void **)&S.p2, H * N * tp * 2 * 2);
     A((void **)&S.a, N * d * es);
     A((void **)&S.g, N * F * es);
     A((void **)&S.u, N * F * es);
@@ -1162,6 +1169,43 @@ extern "C" int rlh_forward_sample(rlh_model *m, rlh_caches *c, const int32_t *to
     return rlh_sample(logits.data(), m->prm.vocab_size, sp, existing_tokens, n_existing, u, token, prob);
 }
 
+// One greedy decode step: the token step for the token in the device state, then argmax + advance.  With
+// RLLAMA_HIP_DECODE_GRAPH=1 the step is captured once per attention grid shape (the only launch parameter that depends on
+// the host's view of the position) and replayed as a graph.
+static int enqueue_decode_step(rlh_model *m, rlh_caches *c, int T_host) {
+    const char *env = getenv("RLLAMA_HIP_DECODE_GRAPH"); // read per call: a process may switch it between calls
+    const bool use_graph = env != nullptr && atoi(env) != 0;
+    hipStream_t st = m->ctx->stream;
+    if (!use_graph) {
+        int rc = enqueue_token_step(m, c, T_host, true);
+        if (rc != RLH_OK) return rc;
+        HIP_TRY(launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st));
+        return RLH_OK;
+    }
+    const int key = attn_splits(m, T_host);
+    auto it = c->step_graphs.find(key);
+    if (it == c->step_graphs.end()) {
+        hipGraph_t graph = nullptr;
+        HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        int rc = enqueue_token_step(m, c, T_host, true);
+        hipError_t e = rc == RLH_OK ? launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st) : hipSuccess;
+        hipError_t e2 = hipStreamEndCapture(st, &graph);
+        if (rc != RLH_OK || e != hipSuccess || e2 != hipSuccess) {
+            if (graph) (void)hipGraphDestroy(graph);
+            if (rc != RLH_OK) return rc;
+            HIP_TRY(e);
+            HIP_TRY(e2);
+        }
+        hipGraphExec_t exec = nullptr;
+        hipError_t e3 = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        HIP_TRY(e3);
+        it = c->step_graphs.emplace(key, exec).first;
+    }
+    HIP_TRY(hipGraphLaunch(it->second, st));
+    return RLH_OK;
+}
+
 extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *prompt, int n_prompt, int n_new, int32_t *out_tokens,
                                    float *ms_first, float *ms_per_token) {
     int rc = check_forward_args(m, c, prompt, n_prompt, 0, "rlh_generate_greedy");
@@ -1188,8 +1232,7 @@ extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *p
     if (rc == RLH_OK && e == hipSuccess) e = hipEventRecord(e1, st);
     for (int i = 1; rc == RLH_OK && e == hipSuccess && i < n_new; i++) {
         // the new token sits at position n_prompt + i - 1; attention spans n_prompt + i positions
-        rc = enqueue_token_step(m, c, n_prompt + i, true);
-        if (rc == RLH_OK) e = launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st);
+        rc = enqueue_decode_step(m, c, n_prompt + i);
     }
     if (rc == RLH_OK && e == hipSuccess) e = hipEventRecord(e2, st);
     if (rc == RLH_OK && e == hipSuccess) e = hipMemcpyAsync(out_tokens, m->out_tokens, sizeof(int32_t) * (size_t)n_new, hipMemcpyDeviceToHost, st);
@@ -1229,8 +1272,7 @@ extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32
     if (e == hipSuccess) e = launch_reset_out(m->state, st);
     if (e == hipSuccess) e = hipEventRecord(e0, st);
     for (int i = 0; rc == RLH_OK && e == hipSuccess && i < n_steps; i++) {
-        rc = enqueue_token_step(m, c, m->next_pos + i + 1, true);
-        if (rc == RLH_OK) e = launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st);
+        rc = enqueue_decode_step(m, c, m->next_pos + i + 1);
     }
     if (rc == RLH_OK && e == hipSuccess) e = hipEventRecord(e1, st);
     if (rc == RLH_OK && e == hipSuccess) e = hipMemcpyAsync(out_tokens, m->out_tokens, sizeof(int32_t) * (size_t)n_steps, hipMemcpyDeviceToHost, st);
