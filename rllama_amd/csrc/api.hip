@@ -10,6 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -123,6 +124,7 @@ struct rlh_model {
     bool prefill_attn_fused = !(getenv("RLLAMA_HIP_PREFILL_ATTN") && !strcmp(getenv("RLLAMA_HIP_PREFILL_ATTN"), "gemm"));
     int prefill_attn_order = getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER") ? atoi(getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER")) : 2;
     // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
+    uint64_t uid = 0;   // unique per created model: a later model at the same address is still another model
     int next_pos = -1;
     rlh_caches *greedy_caches = nullptr;
 };
@@ -130,6 +132,7 @@ struct rlh_model {
 struct rlh_caches {
     rlh_ctx *ctx = nullptr;
     const rlh_model *model = nullptr; // identity only: never dereferenced (the model may be freed first)
+    uint64_t model_uid = 0;
     int n_layers = 0, n_heads = 0, head_dim = 0, max_seq_len = 0;
     void *k = nullptr, *v = nullptr;
     size_t bytes_each = 0;
@@ -266,6 +269,8 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
         return fail(RLH_ERR_UNSUPPORTED, "rlh_model_create: activation vector of %zu bytes does not fit in LDS", lds_need);
     }
     rlh_model *m = new rlh_model();
+    static std::atomic<uint64_t> next_uid{1};
+    m->uid = next_uid.fetch_add(1);
     m->ctx = ctx;
     m->prm = *prm;
     m->prm.percentage_to_gpu = clamp_percentage(prm->percentage_to_gpu);
@@ -552,6 +557,7 @@ extern "C" int rlh_caches_create(rlh_model *m, rlh_caches **out) {
     rlh_caches *c = new rlh_caches();
     c->ctx = m->ctx;
     c->model = m;
+    c->model_uid = m->uid;
     c->n_layers = m->prm.n_layers;
     c->n_heads = m->prm.n_heads;
     c->head_dim = m->head_dim;
@@ -580,6 +586,7 @@ extern "C" int rlh_caches_true_clone(const rlh_caches *src, rlh_caches **out) {
     CtxLock lock(ctx);
     rlh_caches *c = new rlh_caches(*src);
     c->k = c->v = nullptr;
+    c->step_graphs.clear(); // captured steps hold the source's cache addresses: the clone captures its own
     hipError_t e = hipMalloc(&c->k, c->bytes_each);
     if (e == hipSuccess) e = hipMalloc(&c->v, c->bytes_each);
     if (e == hipSuccess) e = hipMemcpyAsync(c->k, src->k, c->bytes_each, hipMemcpyDeviceToDevice, ctx->stream);
@@ -1089,7 +1096,7 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
 
 static int check_forward_args(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, const char *who) {
     if (!m || !c || !tokens) return fail(RLH_ERR_INVALID, "%s: NULL argument", who);
-    if (c->model != m) return fail(RLH_ERR_STATE, "%s: caches belong to another model", who);
+    if (c->model != m || c->model_uid != m->uid) return fail(RLH_ERR_STATE, "%s: caches belong to another model", who);
     if (!model_ready(m)) return fail(RLH_ERR_STATE, "%s: model has tensors that were never set", who);
     if (n < 1) return fail(RLH_ERR_INVALID, "%s: n must be >= 1", who);
     if (n > 1 && start_pos != 0) {
@@ -1254,7 +1261,7 @@ extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *p
 
 extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32_t *out_tokens, float *ms_total) {
     if (!m || !c || !out_tokens || n_steps < 1) return fail(RLH_ERR_INVALID, "rlh_decode_greedy: bad argument");
-    if (c->model != m) return fail(RLH_ERR_STATE, "rlh_decode_greedy: caches belong to another model");
+    if (c->model != m || c->model_uid != m->uid) return fail(RLH_ERR_STATE, "rlh_decode_greedy: caches belong to another model");
     if (m->next_pos < 0 || m->greedy_caches != c) {
         return fail(RLH_ERR_STATE, "rlh_decode_greedy: no sampled token on the device for these caches (call rlh_forward_greedy or rlh_generate_greedy first)");
     }
@@ -1295,7 +1302,7 @@ extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32
 // ------------------------------------------------------------------------------------------------
 extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int T, int iters, float *us_per_launch, uint64_t *bytes_per_launch) {
     if (!m || !c || !us_per_launch || iters < 1) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad argument");
-    if (c->model != m) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: caches belong to another model");
+    if (c->model != m || c->model_uid != m->uid) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: caches belong to another model");
     if (!model_ready(m)) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: model has tensors that were never set");
     if (T < 1 || T > m->prm.max_seq_len || which < kStepQkv || which > kStepHead) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad T or kernel id");
     CtxLock lock(m->ctx);

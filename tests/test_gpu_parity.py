@@ -486,6 +486,9 @@ def test_decode_step_graph_replay(ctx, monkeypatch):
         gm.forward([5], 17, other)
         # token want[lo - 1] sits at position 248 + lo - 1; forwarding it again yields want[lo] and re-seeds the greedy state
         assert gm.forward_greedy([int(want[lo - 1])], 248 + lo - 1, c) == want[lo]
+        if lo == 40:
+            c = c.true_clone()                               # a clone replays its own captures, not its source's
+            assert gm.forward_greedy([int(want[lo - 1])], 248 + lo - 1, c) == want[lo]
         ids, _ = gm.decode_greedy(19, c)
         assert np.array_equal(ids, want[lo + 1:lo + 20])
     gm.free()
