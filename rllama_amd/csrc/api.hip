@@ -88,8 +88,10 @@ struct PrefillScratch {
     // q2: rows [q hi | q lo] of 2 head_dim halves; p2: rows [P hi | P lo] of 2 t_pad halves (one GEMM sums both parts)
     void *xn = nullptr, *qkv = nullptr, *q2 = nullptr, *v_t = nullptr, *p2 = nullptr, *a = nullptr;
     void *g = nullptr, *u = nullptr, *mm = nullptr;
+    void *gemm_ws = nullptr; // fp32 partial sums of split-K products (short prompts)
+    static constexpr size_t kGemmWsBytes = (size_t)64 << 20;
     void release() {
-        void *all[] = {x, h, scores, xn, qkv, q2, v_t, p2, a, g, u, mm};
+        void *all[] = {x, h, scores, xn, qkv, q2, v_t, p2, a, g, u, mm, gemm_ws};
         for (void *b : all)
             if (b) (void)hipFree(b);
         *this = PrefillScratch();
@@ -825,6 +827,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     A((void **)&S.g, N * F * es);
     A((void **)&S.u, N * F * es);
     A((void **)&S.mm, N * F * es);
+    if (es == 2) A((void **)&S.gemm_ws, PrefillScratch::kGemmWsBytes);
     if (e == hipSuccess) e = hipStreamSynchronize(m->ctx->stream);
     if (e != hipSuccess) {
         S.release();
@@ -864,6 +867,8 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         g.ldb = ldb;
         g.ldc = ldc;
         g.batch = 1;
+        g.workspace = S.gemm_ws;
+        g.workspace_bytes = PrefillScratch::kGemmWsBytes;
         HIP_TRY(launch_gemm_f16(g, epi, st));
         return RLH_OK;
     };

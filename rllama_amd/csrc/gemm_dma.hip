@@ -53,12 +53,22 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     const half_t *A = p.a + zb * p.stride_a * kE;
     const half_t *B = p.b + zb * p.stride_b * kE;
     const int M = p.m, N = p.n, K = p.k * kE;          // K, segments and k offsets below are in halves
+    // split_k > 1: grid.z counts K ranges of one product, not batch items (strides of a and b are 0 then): range z takes
+    // K-tiles [z q + min(z, r), ...) of the K / kBK = split_k q + r tiles, one more for z < r; C item z gets its partial sum
+    int split_tiles = -1;
+    if (p.split_k > 1) {
+        const int total = K / kBK, q = total / p.split_k, r = total % p.split_k, z = (int)blockIdx.z;
+        split_tiles = q + (z < r ? 1 : 0);
+        const int skip = (z * q + min(z, r)) * kBK;
+        A += skip;
+        B += skip;
+    }
     if (p.causal == 1 && bn0 > bm0 + kBM - 1) return; // the whole tile lies above the diagonal (uniform for the workgroup)
     // K-tiles: n_seg segments of tps tiles each; A's k runs on from segment to segment, B's starts over
     const int seg_len = p.k_seg > 0 ? p.k_seg * kE : K;
     const int seg_used = p.causal == 2 ? min(seg_len, ((bm0 + kBM) * kE + kBK - 1) / kBK * kBK) : seg_len;
     const int tps = seg_used / kBK;
-    const int n_kt = (K / seg_len) * tps;
+    const int n_kt = split_tiles >= 0 ? split_tiles : (K / seg_len) * tps;
 
     // ---- staging: a stage holds rows 0 .. kBM-1 of A then rows 0 .. kBN-1 of B, kRowBytes each.  Load i of
     //      wavefront w moves row group i * kWaves + w; lane l of a group: row l / kCpr, physical chunk l % kCpr.
@@ -328,8 +338,86 @@ static int choose_tile(const GemmParams &p) {
     return best;
 }
 
-hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s) {
-    if (!gemm_f16_dma_supported(p) || p.m <= 0 || p.n <= 0 || p.batch < 1) return hipErrorInvalidValue;
+// Second step of a split-K product: C = epilogue(sum over the split_k partial sums, in the order of the splits).
+template <int kEpi>
+__global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int splits) {
+    const size_t per = (size_t)p.m * p.ldc;
+    const int n4 = p.n / 4; // n is a multiple of 4 here
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (size_t)p.m * n4; i += (size_t)gridDim.x * blockDim.x) {
+        const int r = (int)(i / n4), c = (int)(i % n4) * 4;
+        const size_t off = (size_t)r * p.ldc + c;
+        float4_t acc = *reinterpret_cast<const float4_t *>(partial + off);
+        for (int z = 1; z < splits; z++) acc += *reinterpret_cast<const float4_t *>(partial + z * per + off);
+        if constexpr (kEpi == kGemmEpiF16) {
+            typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
+            half4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = (half_t)acc[e]; // tensor.rs:1623-1643
+            *reinterpret_cast<half4_t *>(reinterpret_cast<half_t *>(p.c) + off) = o;
+        } else if constexpr (kEpi == kGemmEpiF32) {
+            float4_t *dst = reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.c) + off);
+            *dst = p.accumulate ? *dst + acc : acc;
+        } else {
+            const float4_t res = *reinterpret_cast<const float4_t *>(p.residual + off);
+            float4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = res[e] + f16r(acc[e]);
+            *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.c) + off) = o;
+        }
+    }
+}
+
+// Products with few output tiles (few prompt rows) leave most compute units without a workgroup, and what bounds them is
+// streaming the weights once: the K range is then cut into split_k pieces that run as separate workgroups (more weight bytes
+// in flight, every compute unit busy), their fp32 partial sums go to the caller's workspace and a second small kernel adds
+// them and applies the epilogue.  Returns 1 for "run as one product".
+static int choose_split_k(const GemmParams &p, int tile) {
+    if (p.workspace == nullptr || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.f32_operands) return 1;
+    if (tile != 0 || (p.n % 4) != 0 || (p.ldc % 4) != 0 || p.k % 64 != 0) return 1;
+    static const int forced = getenv("RLLAMA_HIP_GEMM_SPLIT_K") ? atoi(getenv("RLLAMA_HIP_GEMM_SPLIT_K")) : 0;
+    const int n_cu = device_compute_units();
+    const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128);
+    const int k_tiles = p.k / 64;
+    if (blocks * 2 > n_cu && forced <= 1) return 1;       // at least half the compute units have a tile already
+    long s = forced > 1 ? forced : (n_cu + blocks - 1) / blocks;
+    if (s > k_tiles / 4) s = k_tiles / 4;                  // at least 4 K-tiles per piece
+    const size_t per = (size_t)p.m * p.ldc * sizeof(float);
+    if (per > 0 && (size_t)s * per > p.workspace_bytes) s = (long)(p.workspace_bytes / per);
+    return s < 2 ? 1 : (int)s;
+}
+
+template <int kEpi>
+static hipError_t launch_split_finish(const GemmParams &p, int splits, hipStream_t s) {
+    const size_t work = (size_t)p.m * (p.n / 4);
+    const unsigned blocks = (unsigned)((work + 255) / 256 < 4096 ? (work + 255) / 256 : 4096);
+    hipLaunchKernelGGL(gemm_split_finish_kernel<kEpi>, dim3(blocks), dim3(256), 0, s, p, (const float *)p.workspace, splits);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t s) {
+    if (!gemm_f16_dma_supported(p_in) || p_in.m <= 0 || p_in.n <= 0 || p_in.batch < 1) return hipErrorInvalidValue;
+    if (epilogue == kGemmEpiResAddF32 && (p_in.residual == nullptr || p_in.batch != 1)) return hipErrorInvalidValue;
+    const int splits = choose_split_k(p_in, choose_tile(p_in));
+    if (splits > 1) {
+        GemmParams q = p_in;            // the partial sums: split_k pieces as grid.z, fp32 store, C item z = workspace slice z
+        q.c = p_in.workspace;
+        q.residual = nullptr;
+        q.accumulate = 0;
+        q.split_k = splits;
+        q.batch = splits;
+        q.stride_a = q.stride_b = 0;
+        q.stride_c = (size_t)p_in.m * p_in.ldc;
+        q.workspace = nullptr;
+        hipError_t e = launch_gemm_f16_dma(q, kGemmEpiF32, s);
+        if (e != hipSuccess) return e;
+        switch (epilogue) {
+        case kGemmEpiF16: return launch_split_finish<kGemmEpiF16>(p_in, splits, s);
+        case kGemmEpiF32: return launch_split_finish<kGemmEpiF32>(p_in, splits, s);
+        case kGemmEpiResAddF32: return launch_split_finish<kGemmEpiResAddF32>(p_in, splits, s);
+        default: return hipErrorInvalidValue;
+        }
+    }
+    const GemmParams &p = p_in;
     int tile = choose_tile(p);
     if (tile == 0) {
         // With at most one workgroup per compute unit anyway, the LDS that a second one would need buys a deeper load

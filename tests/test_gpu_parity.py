@@ -208,6 +208,20 @@ def test_prefill_fused_attention_head_dims(ctx, n_heads, n, cap):
     gm.free()
 
 
+def test_prefill_short_prompt_split_k(ctx):
+    """Few prompt rows leave few output tiles, so the projections run split along K (uneven pieces: 22 K-tiles over 5
+    workgroups for w2) with a second kernel that adds the partial sums and applies the epilogue; against the oracle."""
+    shape = Shape(dim=512, n_layers=2, n_heads=4, ffn_hidden=1408, vocab_size=64, max_seq_len=128)
+    W = synth_weights(shape, seed=47, std=0.05, norm_ones=False)
+    toks = np.random.default_rng(48).integers(0, shape.vocab_size, 101)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    for n in (100, 5):
+        oc, gc = om.make_caches(), gm.make_caches()
+        assert max_rel_err(gm.forward(toks[:n], 0, gc), om.forward(toks[:n], 0, oc)) < TOL_F16
+        assert max_rel_err(gm.forward(toks[n:n + 1], n, gc), om.forward(toks[n:n + 1], n, oc)) < TOL_F16
+    gm.free()
+
+
 def test_prefill_long_prompt_causal_tiles(ctx):
     """A prompt long enough that the score matrix spans several GEMM tiles per head (tiles above the diagonal are
     skipped, the probability product stops at the diagonal) on the large-tile path; compared with the oracle."""
