@@ -825,7 +825,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     if (gemm_attention && es == 2) A((void **)&S.p2, H * N * tp * 2 * 2);
     A((void **)&S.a, N * d * es);
     A((void **)&S.g, N * F * es);
-    A((void **)&S.u, N * F * es);
+    if (es == 4) A((void **)&S.u, N * F * es); // f16 mode: w3's epilogue consumes its product on the spot
     A((void **)&S.mm, N * F * es);
     if (es == 2) A((void **)&S.gemm_ws, PrefillScratch::kGemmWsBytes);
     if (e == hipSuccess) e = hipStreamSynchronize(m->ctx->stream);
@@ -854,12 +854,14 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));
     HIP_TRY(launch_embed_rows(m->tok_emb.p, m->tok_emb.f16, m->prompt_dev, n, d, S.x, st));
     const size_t layer_elems = (size_t)H * P.max_seq_len * hd;
-    auto gemm = [&](const void *a, int lda, const void *b, int ldb, void *cc, int ldc, int mm, int nn, int kk, int epi, const float *res) -> int {
+    auto gemm = [&](const void *a, int lda, const void *b, int ldb, void *cc, int ldc, int mm, int nn, int kk, int epi, const float *res,
+                    const void *gate = nullptr) -> int {
         GemmParams g{};
         g.a = (const _Float16 *)a;
         g.b = (const _Float16 *)b;
         g.c = cc;
         g.residual = res;
+        g.gate = (const _Float16 *)gate;
         g.m = mm;
         g.n = nn;
         g.k = kk;
@@ -961,8 +963,8 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         if ((rc = gemm(S.a, d, L.wo.p, d, S.h, d, n, d, d, kGemmEpiResAddF32, S.x)) != RLH_OK) return rc;     // h = x + wo(att)
         HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.h, (const float *)L.ffn_norm.p, n, d, eps, st));
         if ((rc = gemm(S.xn, d, L.w1.p, d, S.g, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
-        if ((rc = gemm(S.xn, d, L.w3.p, d, S.u, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
-        HIP_TRY(launch_silu_mul_f16(S.g, S.u, S.mm, (size_t)n * F, st));
+        // w3's epilogue applies SiLU(w1 x) * (w3 x) and the f16 rounding points of transformer.rs:557-565 in place of a pass of its own
+        if ((rc = gemm(S.xn, d, L.w3.p, d, S.mm, F, n, F, d, kGemmEpiSiluGateF16, nullptr, S.g)) != RLH_OK) return rc;
         if ((rc = gemm(S.mm, F, L.w2.p, F, S.x, d, n, d, F, kGemmEpiResAddF32, S.h)) != RLH_OK) return rc;    // x = h + w2(...)
     }
     // final norm + output head on the last row only (transformer.rs:378-381)

@@ -117,6 +117,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_f16_kernel(GemmParams p) {
                     } else if constexpr (kEpi == kGemmEpiF32) {
                         float *cp = reinterpret_cast<float *>(p.c) + off;
                         *cp = p.accumulate ? (*cp + val) : val;
+                    } else if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
+                        const float g = (float)p.gate[(size_t)r * p.ldc + c];
+                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)((g / (1.0f + expf(-g))) * f16r(val));
                     } else { // kGemmEpiResAddF32: residual add of transformer.rs:442 / :445 on the f16-rounded product
                         reinterpret_cast<float *>(p.c)[off] = p.residual[(size_t)r * p.ldc + c] + f16r(val);
                     }
@@ -143,6 +146,10 @@ hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s) {
     case kGemmEpiResAddF32:
         if (p.residual == nullptr || p.batch != 1) return hipErrorInvalidValue;
         hipLaunchKernelGGL(gemm_f16_kernel<kGemmEpiResAddF32>, grid, dim3(kGemmThreads), 0, s, p);
+        break;
+    case kGemmEpiSiluGateF16:
+        if (p.gate == nullptr || p.batch != 1) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(gemm_f16_kernel<kGemmEpiSiluGateF16>, grid, dim3(kGemmThreads), 0, s, p);
         break;
     default: return hipErrorInvalidValue;
     }

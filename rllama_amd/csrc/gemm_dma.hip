@@ -134,6 +134,25 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                 }
     }
 
+    // SiLU-gate epilogue: the gate values this lane will need (the 16-byte pieces it handles in the row-wise epilogue below)
+    // are fetched now as well, for the same reason.
+    [[maybe_unused]] const bool rows16 = (p.ldc % 8) == 0 && (N % 8) == 0 && ((zb * p.stride_c) % 8) == 0 && (reinterpret_cast<uintptr_t>(p.c) % 16) == 0 &&
+                                         (kEpi != kGemmEpiSiluGateF16 || (reinterpret_cast<uintptr_t>(p.gate) % 16) == 0);
+    constexpr bool kGatePre = kEpi == kGemmEpiSiluGateF16 && kNT <= 3; // the widest tile has no registers to spare for it
+    constexpr int kGateChunks = kGatePre ? 32 * kNT / 8 : 1;
+    [[maybe_unused]] half8_t gate_pre[kGateChunks];
+    if constexpr (kGatePre) {
+        if (rows16) {
+#pragma unroll
+            for (int it = 0; it < kGateChunks; it++) {
+                const int idx = it * 64 + lane;
+                const int rr = idx / kGateChunks, ch = idx - rr * kGateChunks;
+                const int r = bm0 + wm * 64 + rr, c = bn0 + wn * (32 * kNT) + ch * 8;
+                gate_pre[it] = (r < M && c < N) ? *reinterpret_cast<const half8_t *>(p.gate + (size_t)r * p.ldc + c) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            }
+        }
+    }
+
     // operand fragments: lane l supplies row (l % 32), logical chunk 2 * ks + l / 32 of a 32 x 16 slab
     const int frow = lane & 31, fch = lane >> 5;
     int a_off[2], a_sw[2], b_off[kNT], b_sw[kNT];
@@ -217,6 +236,50 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     const int row_in = (lane >> 5) * 4;
     auto out_row = [&](int i, int v) { return bm0 + wm * 64 + i * 32 + (v >> 2) * 8 + row_in + (v & 3); };
     auto out_col = [&](int j) { return bn0 + wn * (32 * kNT) + j * 32 + col_in; };
+    // f16 outputs whose rows are 16-byte aligned go through LDS (the stages are free now): every wavefront lays its 64 x 32 kNT
+    // tile out as rows, then stores whole 16-byte pieces of consecutive columns (and, with the SiLU gate, reads the gate the
+    // same way) instead of one 2-byte element per lane and accumulator register.
+    if constexpr (kEpi == kGemmEpiF16 || kEpi == kGemmEpiSiluGateF16) {
+        if (rows16) { // uniform for the launch
+            constexpr int kTW = 32 * kNT; // tile width of a wavefront
+            constexpr int kPad = (kWaves * 64 * (kTW + 8) * 2 <= kStages * kStageBytes) ? 8 : 0;
+            constexpr int kTS = kTW + kPad; // halves per LDS row
+            static_assert(kWaves * 64 * kTS * 2 <= kStages * kStageBytes, "the output tiles reuse the stages");
+            constexpr int kChunks = kTW / 8;
+            __syncthreads(); // every wavefront has read its last fragments
+            half_t *tile = reinterpret_cast<half_t *>(lds_raw) + wave * (64 * kTS);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < kNT; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        tile[(i * 32 + (v >> 2) * 8 + row_in + (v & 3)) * kTS + j * 32 + col_in] = (half_t)acc[i][j][v]; // tensor.rs:1623-1643
+            half_t *cbase = reinterpret_cast<half_t *>(p.c) + zb * p.stride_c;
+#pragma unroll
+            for (int it = 0; it < kChunks; it++) {
+                const int idx = it * 64 + lane;
+                const int rr = idx / kChunks, ch = idx - rr * kChunks;
+                const int r = bm0 + wm * 64 + rr, c = bn0 + wn * kTW + ch * 8;
+                if (r < M && c < N) {
+                    half8_t o = *reinterpret_cast<const half8_t *>(tile + rr * kTS + ch * 8);
+                    const size_t off = (size_t)r * p.ldc + c;
+                    if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
+                        half8_t g8;
+                        if constexpr (kGatePre) g8 = gate_pre[it];
+                        else g8 = *reinterpret_cast<const half8_t *>(p.gate + off);
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            const float g = (float)g8[e];
+                            o[e] = (half_t)((g / (1.0f + expf(-g))) * (float)o[e]);
+                        }
+                    }
+                    *reinterpret_cast<half8_t *>(cbase + off) = o;
+                }
+            }
+            return;
+        }
+    }
     // What the epilogue adds to (the residual, or C itself when accumulating) is loaded in batches of one column
     // tile: C may alias the residual, so a load issued between the stores would wait for the store before it.
     [[maybe_unused]] const float *prev_src = nullptr;
@@ -229,6 +292,14 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         if constexpr (kEarlyResidual) {
             prev[0] = early[0][j];
             prev[1] = early[1][j];
+        } else if constexpr (kEpi == kGemmEpiSiluGateF16) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = out_row(i, v);
+                    prev[i][v] = (r < M && c < N) ? (float)p.gate[(size_t)r * p.ldc + c] : 0.0f;
+                }
         } else if constexpr (kEpi != kGemmEpiF16) {
 #pragma unroll
             for (int i = 0; i < 2; i++)
@@ -250,6 +321,9 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                         reinterpret_cast<half_t *>(p.c)[off] = (half_t)val; // tensor.rs:1623-1643
                     } else if constexpr (kEpi == kGemmEpiF32) {
                         reinterpret_cast<float *>(p.c)[off] = prev[i][v] + val;
+                    } else if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
+                        const float g = prev[i][v];
+                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)((g / (1.0f + expf(-g))) * f16r(val));
                     } else { // kGemmEpiResAddF32: residual add of transformer.rs:442 / :445 on the f16-rounded product
                         reinterpret_cast<float *>(p.c)[off] = prev[i][v] + f16r(val);
                     }
@@ -357,6 +431,16 @@ __global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int
         } else if constexpr (kEpi == kGemmEpiF32) {
             float4_t *dst = reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.c) + off);
             *dst = p.accumulate ? *dst + acc : acc;
+        } else if constexpr (kEpi == kGemmEpiSiluGateF16) {
+            typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
+            const half4_t g4 = *reinterpret_cast<const half4_t *>(p.gate + off);
+            half4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float g = (float)g4[e];
+                o[e] = (half_t)((g / (1.0f + expf(-g))) * f16r(acc[e]));
+            }
+            *reinterpret_cast<half4_t *>(reinterpret_cast<half_t *>(p.c) + off) = o;
         } else {
             const float4_t res = *reinterpret_cast<const float4_t *>(p.residual + off);
             float4_t o;
@@ -397,6 +481,7 @@ static hipError_t launch_split_finish(const GemmParams &p, int splits, hipStream
 hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t s) {
     if (!gemm_f16_dma_supported(p_in) || p_in.m <= 0 || p_in.n <= 0 || p_in.batch < 1) return hipErrorInvalidValue;
     if (epilogue == kGemmEpiResAddF32 && (p_in.residual == nullptr || p_in.batch != 1)) return hipErrorInvalidValue;
+    if (epilogue == kGemmEpiSiluGateF16 && (p_in.gate == nullptr || p_in.batch != 1 || p_in.f32_operands)) return hipErrorInvalidValue;
     const int splits = choose_split_k(p_in, choose_tile(p_in));
     if (splits > 1) {
         GemmParams q = p_in;            // the partial sums: split_k pieces as grid.z, fp32 store, C item z = workspace slice z
@@ -414,6 +499,7 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         case kGemmEpiF16: return launch_split_finish<kGemmEpiF16>(p_in, splits, s);
         case kGemmEpiF32: return launch_split_finish<kGemmEpiF32>(p_in, splits, s);
         case kGemmEpiResAddF32: return launch_split_finish<kGemmEpiResAddF32>(p_in, splits, s);
+        case kGemmEpiSiluGateF16: return launch_split_finish<kGemmEpiSiluGateF16>(p_in, splits, s);
         default: return hipErrorInvalidValue;
         }
     }
@@ -435,6 +521,7 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
     case kGemmEpiResAddF32:
         if (p.residual == nullptr || p.batch != 1) return hipErrorInvalidValue;
         return launch_dma_epi<kGemmEpiResAddF32>(p, tile, s);
+    case kGemmEpiSiluGateF16: return launch_dma_epi<kGemmEpiSiluGateF16>(p, tile, s);
     default: return hipErrorInvalidValue;
     }
 }

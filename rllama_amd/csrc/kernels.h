@@ -75,7 +75,8 @@ hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s);
 enum GemmEpilogue {
     kGemmEpiF16 = 0,        // C f16 = round(acc)                      (projection outputs, tensor.rs:1623-1643)
     kGemmEpiF32 = 1,        // C f32 = acc, or += acc when accumulate  (attention scores / P.V partial products)
-    kGemmEpiResAddF32 = 2   // C f32 = residual + f16r(acc)            (wo and w2 followed by transformer.rs:442 / :445)
+    kGemmEpiResAddF32 = 2,  // C f32 = residual + f16r(acc)            (wo and w2 followed by transformer.rs:442 / :445)
+    kGemmEpiSiluGateF16 = 3 // C f16 = round(silu(gate) * f16r(acc))   (w3 with w1's f16 output as the gate: transformer.rs:557-565)
 };
 
 struct GemmParams {
@@ -83,6 +84,7 @@ struct GemmParams {
     const _Float16 *b;      // [n x k], row stride ldb
     void *c;                // [m x n], row stride ldc
     const float *residual;  // kGemmEpiResAddF32: [m x n], row stride ldc
+    const _Float16 *gate;   // kGemmEpiSiluGateF16: [m x n], row stride ldc
     int m, n, k;
     int lda, ldb, ldc;
     int batch;              // grid.z; element strides between batch items:
@@ -151,7 +153,6 @@ hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int 
 hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s);
 // scores rows are t_pad floats apart, the probability rows (hi and lo alike) p_stride halves
 hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int p_stride, int head_dim, hipStream_t s);
-hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s);
 
 hipError_t launch_embed(const void *table, int table_f16, int dim, const DecodeState *state, float *x, hipStream_t s);
 // argmax with TokenSampler's top_k = 1 behaviour (token_sampler.rs:112-147); writes state->token, appends to

@@ -258,33 +258,4 @@ hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, in
     return hipGetLastError();
 }
 
-// m = f16r(silu(g) * u) on f16 tensors (transformer.rs:557-565; tensor.rs:822-832, 722-734), 8 elements per thread
-__global__ void silu_mul_f16_kernel(const half_t *g, const half_t *u, half_t *m, size_t total) {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const size_t n8 = total / 8;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
-        const half8_t gv = reinterpret_cast<const half8_t *>(g)[i], uv = reinterpret_cast<const half8_t *>(u)[i];
-        half8_t o;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const float x = (float)gv[e];
-            const float sg = x / (1.0f + expf(-x));
-            o[e] = (half_t)(sg * (float)uv[e]);
-        }
-        reinterpret_cast<half8_t *>(m)[i] = o;
-    }
-    for (size_t i = n8 * 8 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const float x = (float)g[i];
-        const float sg = x / (1.0f + expf(-x));
-        m[i] = (half_t)(sg * (float)u[i]);
-    }
-}
-
-hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s) {
-    const size_t work = (total + 7) / 8;
-    const int blocks = (int)((work + 255) / 256 < 8192 ? (work + 255) / 256 : 8192);
-    hipLaunchKernelGGL(silu_mul_f16_kernel, dim3(blocks > 0 ? blocks : 1), dim3(256), 0, s, (const half_t *)g, (const half_t *)u, (half_t *)m, total);
-    return hipGetLastError();
-}
-
 } // namespace rlh

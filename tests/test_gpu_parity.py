@@ -222,6 +222,19 @@ def test_prefill_short_prompt_split_k(ctx):
     gm.free()
 
 
+def test_prefill_wide_ffn_largest_tile(ctx):
+    """An FFN wide enough that w1 / w3 (1024 x 16384 outputs) take the 256 x 256 tile, whose SiLU-gate epilogue reads the gate
+    in the epilogue instead of ahead of the K loop; against the oracle."""
+    shape = Shape(dim=256, n_layers=1, n_heads=2, ffn_hidden=16384, vocab_size=64, max_seq_len=1024)
+    W = synth_weights(shape, seed=49, std=0.03, norm_ones=False)
+    toks = np.random.default_rng(50).integers(0, shape.vocab_size, 1024)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    want = om.forward(toks, 0, om.make_caches())
+    got = gm.forward(toks, 0, gm.make_caches())
+    assert max_rel_err(got, want) < TOL_F16, max_rel_err(got, want)
+    gm.free()
+
+
 def test_prefill_long_prompt_causal_tiles(ctx):
     """A prompt long enough that the score matrix spans several GEMM tiles per head (tiles above the diagonal are
     skipped, the probability product stops at the diagonal) on the large-tile path; compared with the oracle."""
