@@ -175,6 +175,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // of K-step s run (two fragment sets, selected by the parity of the unrolled K-step); the tile change sits in
     // the middle of the last K-step's MFMAs so that the barrier and the LDS latency behind it stay covered.
     constexpr int kKS = kBK / 16;
+    constexpr int kSplitJ = kNT / 2; // column tiles of the last K-step whose MFMAs run before the tile change (0 .. kNT measured alike)
     static_assert(kKS % 2 == 0, "fragment sets alternate by K-step parity");
     half8_t af[2][2], bf[2][kNT];
     auto mma = [&](const half8_t &a, const half8_t &b, float16_t &c) {
@@ -210,9 +211,20 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                 for (int j = 0; j < kNT; j++)
 #pragma unroll
                     for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                {   // order within the step: an LDS fragment read of the next step behind each of the first MFMAs of this one,
+                    // so that the reads are in flight under the matrix pipe and none is left to wait for when the next step
+                    // begins (left to itself the scheduler issues the reads at the end of the step and the MFMAs wait for them)
+                    constexpr int kPerMma = kF32 ? 4 : 1; // MFMA instructions per fragment pair
+#pragma unroll
+                    for (int r = 0; r < 2 + kNT; r++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, kPerMma, 0); // MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // DS read
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, (2 * kNT - (2 + kNT)) * kPerMma, 0);
+                }
             } else {
 #pragma unroll
-                for (int j = 0; j < kNT / 2; j++)
+                for (int j = 0; j < kSplitJ; j++)
 #pragma unroll
                     for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
                 __builtin_amdgcn_sched_barrier(0);
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                 read_frags(nxt, lds_raw + ((kt + 1) % kStages) * kStageBytes, 0);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = kNT / 2; j < kNT; j++)
+                for (int j = kSplitJ; j < kNT; j++)
 #pragma unroll
                     for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
             }
