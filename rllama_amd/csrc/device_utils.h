@@ -107,6 +107,13 @@ __device__ __forceinline__ void rope_pair(float re, float im, float2 f, float &o
     oim = p2 + p3;
 }
 
+// SiLU (tensor.rs:822-832: v / (1 + exp(-v))) through the hardware exp2 and reciprocal: about 3e-7 relative from the
+// libm form, i.e. one f16-rounded product in a few thousand lands on the neighbouring f16 value.  Used where the call
+// sits in a GEMM epilogue that every wavefront of the chip runs at the same time (there the libm form costs 6 us per launch).
+__device__ __forceinline__ float silu_fast(float v) {
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.44269504088896340736f));
+}
+
 // One direct-to-LDS load: lane l's 16 bytes at `src` land at LDS byte address dst + 16 l (dst is wave-uniform and
 // travels in M0).  Written as inline assembly on purpose: through the builtin the compiler tracks the load as an LDS
 // write and puts s_waitcnt vmcnt(0) in front of every LDS read, which would also wait for the prefetched K-tiles;

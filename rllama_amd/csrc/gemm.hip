@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_f16_kernel(GemmParams p) {
                         *cp = p.accumulate ? (*cp + val) : val;
                     } else if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
                         const float g = (float)p.gate[(size_t)r * p.ldc + c];
-                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)((g / (1.0f + expf(-g))) * f16r(val));
+                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)(silu_fast(g) * f16r(val));
                     } else { // kGemmEpiResAddF32: residual add of transformer.rs:442 / :445 on the f16-rounded product
                         reinterpret_cast<float *>(p.c)[off] = p.residual[(size_t)r * p.ldc + c] + f16r(val);
                     }

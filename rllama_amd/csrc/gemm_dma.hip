@@ -283,7 +283,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
                         for (int e = 0; e < 8; e++) {
                             const float g = (float)g8[e];
-                            o[e] = (half_t)((g / (1.0f + expf(-g))) * (float)o[e]);
+                            o[e] = (half_t)(silu_fast(g) * (float)o[e]);
                         }
                     }
                     *reinterpret_cast<half8_t *>(cbase + off) = o;
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                         reinterpret_cast<float *>(p.c)[off] = prev[i][v] + val;
                     } else if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
                         const float g = prev[i][v];
-                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)((g / (1.0f + expf(-g))) * f16r(val));
+                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)(silu_fast(g) * f16r(val));
                     } else { // kGemmEpiResAddF32: residual add of transformer.rs:442 / :445 on the f16-rounded product
                         reinterpret_cast<float *>(p.c)[off] = prev[i][v] + f16r(val);
                     }
@@ -450,7 +450,7 @@ __global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const float g = (float)g4[e];
-                o[e] = (half_t)((g / (1.0f + expf(-g))) * f16r(acc[e]));
+                o[e] = (half_t)(silu_fast(g) * f16r(acc[e]));
             }
             *reinterpret_cast<half4_t *>(reinterpret_cast<half_t *>(p.c) + off) = o;
         } else {
