@@ -474,7 +474,11 @@ static int choose_split_k(const GemmParams &p, int tile) {
     const int n_cu = device_compute_units();
     const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128);
     const int k_tiles = p.k / 64;
-    if (blocks * 2 > n_cu && forced <= 1) return 1;       // at least half the compute units have a tile already
+    // Worth it while the partial sums (pieces x m x n floats, written and read back) stay small beside the weights: up to a
+    // quarter of the compute units covered, or half with at most 32 rows (measured on the 7B shapes: wq|wk|wv / w1 / w3 at 64
+    // to 256 rows are faster unsplit on their 86 - 96 tiles, at 8 rows faster split)
+    const long max_blocks = p.m <= 32 ? n_cu / 2 : n_cu / 4;
+    if (blocks > max_blocks && forced <= 1) return 1;
     long s = forced > 1 ? forced : (n_cu + blocks - 1) / blocks;
     if (s > k_tiles / 4) s = k_tiles / 4;                  // at least 4 K-tiles per piece
     const size_t per = (size_t)p.m * p.ldc * sizeof(float);
