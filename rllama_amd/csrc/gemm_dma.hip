@@ -215,12 +215,14 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                     // so that the reads are in flight under the matrix pipe and none is left to wait for when the next step
                     // begins (left to itself the scheduler issues the reads at the end of the step and the MFMAs wait for them)
                     constexpr int kPerMma = kF32 ? 4 : 1; // MFMA instructions per fragment pair
+                    constexpr int kMmas = 2 * kNT, kReads = 2 + kNT, kPairs = kMmas < kReads ? kMmas : kReads;
 #pragma unroll
-                    for (int r = 0; r < 2 + kNT; r++) {
+                    for (int r = 0; r < kPairs; r++) {
                         __builtin_amdgcn_sched_group_barrier(0x008, kPerMma, 0); // MFMA
                         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // DS read
                     }
-                    __builtin_amdgcn_sched_group_barrier(0x008, (2 * kNT - (2 + kNT)) * kPerMma, 0);
+                    if constexpr (kMmas > kPairs) __builtin_amdgcn_sched_group_barrier(0x008, (kMmas - kPairs) * kPerMma, 0);
+                    if constexpr (kReads > kPairs) __builtin_amdgcn_sched_group_barrier(0x100, kReads - kPairs, 0);
                 }
             } else {
 #pragma unroll
@@ -386,6 +388,7 @@ static hipError_t launch_dma_epi(const GemmParams &p, int tile, hipStream_t s) {
     switch (tile) {
     case 0: return launch_dma<kEpi, 2, 2, 64, 2>(p, s);  // 128 x 128, 64 KiB of LDS: two workgroups per compute unit
     case 4: return launch_dma<kEpi, 2, 2, 64, 4>(p, s);  // 128 x 128, 128 KiB: one workgroup per compute unit, three K-tiles ahead
+    case 5: return launch_dma<kEpi, 2, 1, 64, 6>(p, s);  // 128 x 64, 144 KiB: few rows, so twice the workgroups stream the weights
     case 1: return k64 ? launch_dma<kEpi, 4, 2, 64, 3>(p, s) : launch_dma<kEpi, 4, 2, 32, 4>(p, s);  // 256 x 128
     case 2: return k64 ? launch_dma<kEpi, 4, 3, 64, 2>(p, s) : launch_dma<kEpi, 4, 3, 32, 4>(p, s);  // 256 x 192
     case 3: return k64 ? launch_dma<kEpi, 4, 4, 64, 2>(p, s) : launch_dma<kEpi, 4, 4, 32, 4>(p, s);  // 256 x 256
@@ -474,10 +477,10 @@ static int choose_split_k(const GemmParams &p, int tile) {
     const int n_cu = device_compute_units();
     const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128);
     const int k_tiles = p.k / 64;
-    // Worth it while the partial sums (pieces x m x n floats, written and read back) stay small beside the weights: up to a
-    // quarter of the compute units covered, or half with at most 32 rows (measured on the 7B shapes: wq|wk|wv / w1 / w3 at 64
-    // to 256 rows are faster unsplit on their 86 - 96 tiles, at 8 rows faster split)
-    const long max_blocks = p.m <= 32 ? n_cu / 2 : n_cu / 4;
+    // Worth it while the partial sums (pieces x m x n floats, written and read back) stay small beside the weights: products
+    // whose tiles cover at most a quarter of the compute units (measured on the 7B shapes: wq|wk|wv / w1 / w3 on their 86 - 96
+    // tiles are faster unsplit on the narrower 128 x 64 tile at any row count, wo / w2 on 32 tiles faster split)
+    const long max_blocks = n_cu / 4;
     if (blocks > max_blocks && forced <= 1) return 1;
     long s = forced > 1 ? forced : (n_cu + blocks - 1) / blocks;
     if (s > k_tiles / 4) s = k_tiles / 4;                  // at least 4 K-tiles per piece
@@ -526,6 +529,10 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         // pipeline instead (measured on the wo / w2 products of a 1024-token 7B prefill: 108 -> 85 us per launch).
         const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128) * p.batch;
         if (blocks <= device_compute_units()) tile = 4;
+#ifndef RLH_GEMM_NO_T5
+        // one row tile and few column tiles (a short prompt on a product too large to split): halve the tile width
+        if (!p.f32_operands && p.split_k <= 1 && p.m <= 128 && p.batch == 1 && blocks * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = 5;
+#endif
     }
     if (p.f32_operands) {
         if (epilogue != kGemmEpiF32 || ((p.k * 2) % 64) != 0 || (p.k_seg != 0 && ((p.k_seg * 2) % 64) != 0)) return hipErrorInvalidValue;
