@@ -482,7 +482,9 @@ static int choose_split_k(const GemmParams &p, int tile) {
     // tiles are faster unsplit on the narrower 128 x 64 tile at any row count, wo / w2 on 32 tiles faster split)
     const long max_blocks = n_cu / 4;
     if (blocks > max_blocks && forced <= 1) return 1;
-    long s = forced > 1 ? forced : (n_cu + blocks - 1) / blocks;
+    // a single row tile runs its pieces on the 128 x 64 tile: twice the column tiles, half the pieces, half the partial sums
+    const long tiles = p.m <= 128 ? (long)((p.n + 63) / 64) : blocks;
+    long s = forced > 1 ? forced : (n_cu + tiles - 1) / tiles;
     if (s > k_tiles / 4) s = k_tiles / 4;                  // at least 4 K-tiles per piece
     const size_t per = (size_t)p.m * p.ldc * sizeof(float);
     if (per > 0 && (size_t)s * per > p.workspace_bytes) s = (long)(p.workspace_bytes / per);
@@ -529,10 +531,9 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         // pipeline instead (measured on the wo / w2 products of a 1024-token 7B prefill: 108 -> 85 us per launch).
         const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128) * p.batch;
         if (blocks <= device_compute_units()) tile = 4;
-#ifndef RLH_GEMM_NO_T5
-        // one row tile and few column tiles (a short prompt on a product too large to split): halve the tile width
-        if (!p.f32_operands && p.split_k <= 1 && p.m <= 128 && p.batch == 1 && blocks * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = 5;
-#endif
+        // one row tile and few column tiles (a short prompt): half the tile width, so that twice the workgroups stream the
+        // weights; the pieces of a split product use it too
+        if (!p.f32_operands && p.m <= 128 && (p.batch == 1 || p.split_k > 1) && (long)((p.n + 127) / 128) * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = 5;
     }
     if (p.f32_operands) {
         if (epilogue != kGemmEpiF32 || ((p.k * 2) % 64) != 0 || (p.k_seg != 0 && ((p.k_seg * 2) % 64) != 0)) return hipErrorInvalidValue;
