@@ -521,15 +521,16 @@ def test_decode_step_graph_replay(ctx, monkeypatch):
     gm.free()
 
 
-def test_full_size_7b_properties(ctx):
+@pytest.mark.parametrize("n_prompt", [200, 1100], ids=["200-tokens", "1100-tokens"])
+def test_full_size_7b_properties(ctx, n_prompt):
     """At the full size of the headline configuration (LLaMA-7B shape, f16 mode, synthetic weights) the oracle is out of reach,
     so this checks what holds at any size: the matrix-core prefill and the token-by-token path are the same function (logits
     within the f16-mode tolerance, same greedy continuation), the greedy loop is deterministic, and a true_clone of the caches
     continues exactly like the original."""
     dim, L, H, F, V = 4096, 32, 32, 11008, 32000
-    m = rllama_amd.Transformer(ctx, dim, L, H, F, V, 512, 1e-6, rllama_amd.DataSettings(ctx).force_f16())
+    m = rllama_amd.Transformer(ctx, dim, L, H, F, V, n_prompt + 64, 1e-6, rllama_amd.DataSettings(ctx).force_f16())
     m.fill_synthetic(0, 0.02)
-    prompt = rllama_amd.synth_tokens(0, 200, 3, V)
+    prompt = rllama_amd.synth_tokens(0, n_prompt, 3, V)
     ca, cb = m.make_caches(), m.make_caches()
     a = m.forward(prompt, 0, ca)                       # matrix-core prefill
     m.set_prefill_mode(True)
@@ -540,18 +541,18 @@ def test_full_size_7b_properties(ctx):
     for l in (0, L - 1):                               # the caches the two paths leave agree to f16 rounding noise
         for which in (0, 1):
             ka, kb = ca.read(l, 5, which), cb.read(l, 5, which)
-            assert not np.any(ka[:, 200:]) and not np.any(kb[:, 200:])
+            assert not np.any(ka[:, n_prompt:]) and not np.any(kb[:, n_prompt:])
             # layer 0 sees identical inputs; by the last layer 31 layers of f16 rounding decisions have diverged
             slack = 2e-3 if l == 0 else TOL_F16
-            assert np.all(np.abs(ka[:, :200] - kb[:, :200]) <= 2 * ulp_f16(kb[:, :200]) + slack * np.abs(kb[:, :200]).max())
+            assert np.all(np.abs(ka[:, :n_prompt] - kb[:, :n_prompt]) <= 2 * ulp_f16(kb[:, :n_prompt]) + slack * np.abs(kb[:, :n_prompt]).max())
     c1, c2 = m.make_caches(), m.make_caches()
     ids1, _, _ = m.generate_greedy(prompt, 24, c1)
     ids2, _, _ = m.generate_greedy(prompt, 24, c2)
     assert np.array_equal(ids1, ids2)                  # same kernels, same order of additions: bit-identical runs
     c3 = c2.true_clone()
     nxt = int(ids2[-1])
-    la = m.forward([nxt], 200 + 23, c2)
-    lb = m.forward([nxt], 200 + 23, c3)
+    la = m.forward([nxt], n_prompt + 23, c2)
+    lb = m.forward([nxt], n_prompt + 23, c3)
     assert np.array_equal(la, lb)
     m.free()
 
