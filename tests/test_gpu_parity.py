@@ -208,6 +208,29 @@ def test_prefill_fused_attention_head_dims(ctx, n_heads, n, cap):
     gm.free()
 
 
+def test_prefill_attention_gemm_form_for_large_heads(ctx, monkeypatch):
+    """RLLAMA_HIP_PREFILL_ATTN=gemm (read when a model is created) keeps head_dim 64 / 128 on the two-GEMM form of the
+    prefill attention (hi | lo halves of q and of P as K segments, tiles above the diagonal skipped, V^T in natural key
+    order): same function as the one-kernel form and the oracle."""
+    shape = Shape(dim=256, n_layers=2, n_heads=2, ffn_hidden=512, vocab_size=128, max_seq_len=320)   # head_dim 128
+    W = synth_weights(shape, seed=53, std=0.08, norm_ones=False)
+    toks = np.random.default_rng(54).integers(0, shape.vocab_size, 301)
+    om = make_oracle(shape, W, True)
+    fused = make_gpu(ctx, shape, W, True)
+    monkeypatch.setenv("RLLAMA_HIP_PREFILL_ATTN", "gemm")
+    gemm_form = make_gpu(ctx, shape, W, True)
+    monkeypatch.delenv("RLLAMA_HIP_PREFILL_ATTN")
+    for n in (300, 65):
+        oc, ca, cb = om.make_caches(), fused.make_caches(), gemm_form.make_caches()
+        want = om.forward(toks[:n], 0, oc)
+        a, b = fused.forward(toks[:n], 0, ca), gemm_form.forward(toks[:n], 0, cb)
+        assert max_rel_err(a, want) < TOL_F16 and max_rel_err(b, want) < TOL_F16, (n, max_rel_err(a, want), max_rel_err(b, want))
+        want1 = om.forward(toks[n:n + 1], n, oc)
+        assert max_rel_err(gemm_form.forward(toks[n:n + 1], n, cb), want1) < TOL_F16
+    fused.free()
+    gemm_form.free()
+
+
 def test_prefill_short_prompt_split_k(ctx):
     """Few prompt rows leave few output tiles, so the projections run split along K (uneven pieces: 22 K-tiles over 5
     workgroups for w2) with a second kernel that adds the partial sums and applies the epilogue; against the oracle."""
