@@ -231,6 +231,20 @@ def test_prefill_attention_gemm_form_for_large_heads(ctx, monkeypatch):
     gemm_form.free()
 
 
+def test_prefill_odd_dims_register_staged_gemm(ctx):
+    """dim 48 and ffn 104 are not multiples of the fast GEMM's K-tile, so every product of the multi-token forward (with the
+    SiLU-gate and residual epilogues, and the two attention products at head_dim 16) runs on the register-staged kernel."""
+    shape = Shape(dim=48, n_layers=2, n_heads=3, ffn_hidden=104, vocab_size=50, max_seq_len=40)
+    W = synth_weights(shape, seed=55, std=0.1, norm_ones=False)
+    toks = np.random.default_rng(56).integers(0, shape.vocab_size, 31)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    for n in (30, 3):
+        oc, gc = om.make_caches(), gm.make_caches()
+        assert max_rel_err(gm.forward(toks[:n], 0, gc), om.forward(toks[:n], 0, oc)) < TOL_F16
+        assert max_rel_err(gm.forward(toks[n:n + 1], n, gc), om.forward(toks[n:n + 1], n, oc)) < TOL_F16
+    gm.free()
+
+
 def test_prefill_short_prompt_split_k(ctx):
     """Few prompt rows leave few output tiles, so the projections run split along K (uneven pieces: 22 K-tiles over 5
     workgroups for w2) with a second kernel that adds the partial sums and applies the epilogue; against the oracle."""
