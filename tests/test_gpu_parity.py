@@ -594,6 +594,34 @@ def test_full_size_7b_properties(ctx, n_prompt):
     m.free()
 
 
+@pytest.mark.parametrize("dim,L,H,F,n_prompt", [(5120, 40, 40, 13824, 300), (8192, 80, 64, 22016, 96)], ids=["13B-shape", "65B-shape"])
+def test_full_size_larger_shapes_prefill_equals_token_by_token(ctx, dim, L, H, F, n_prompt):
+    """The 13B and 65B shapes of the other configurations (other GEMM tile choices, split factors and attention grids than 7B):
+    the matrix-core prefill against the token-by-token path.  Two valid orders of fp32 additions flip f16 rounding decisions
+    at seven places per layer, and with random weights the difference random-walks with depth (measured at 65B: mean cache
+    difference / rms 5e-4 after layer 1, 2.6e-3 after 10, 6.7e-3 after 40, 1.0e-2 after 79; logits 1.6e-2), so the bounds
+    scale with the square root of the depth; a wrong tile or split would show as a jump at the layer where it happens."""
+    V = 32000
+    m = rllama_amd.Transformer(ctx, dim, L, H, F, V, n_prompt + 16, 1e-6, rllama_amd.DataSettings(ctx).force_f16())
+    m.fill_synthetic(0, 0.02)
+    prompt = rllama_amd.synth_tokens(0, n_prompt, 3, V)
+    ca, cb = m.make_caches(), m.make_caches()
+    a = m.forward(prompt, 0, ca)
+    m.set_prefill_mode(True)
+    b = m.forward(prompt, 0, cb)
+    m.set_prefill_mode(False)
+    tol = 1.5 * TOL_F16 * (L / 32) ** 0.5
+    assert max_rel_err(a, b) < tol, max_rel_err(a, b)
+    for l in (0, 1, L // 4, L // 2, L - 1):
+        for which in (0, 1):
+            ka, kb = ca.read(l, 5, which)[:, :n_prompt], cb.read(l, 5, which)[:, :n_prompt]
+            noise = float(np.abs(ka - kb).mean() / np.sqrt((kb.astype(np.float64) ** 2).mean()))
+            assert noise < 2e-3 * (l + 1) ** 0.5, (l, which, noise)
+    nxt = [int(np.argmax(a[1:])) + 1]
+    assert max_rel_err(m.forward(nxt, n_prompt, ca), m.forward(nxt, n_prompt, cb)) < tol
+    m.free()
+
+
 def _checkpoint_tensors(shape, W):
     """The reference's tensor names -> f16 bits, from a weight dict of common.synth_weights (norms rounded to f16)."""
     names = {rllama_amd.TOK_EMB: "tok_embeddings.weight", rllama_amd.NORM: "norm.weight", rllama_amd.OUTPUT: "output.weight"}
