@@ -428,7 +428,7 @@ static int choose_tile(const GemmParams &p) {
     if (forced == 0 && k_halves % 64 == 0) return 0;
     const int n_cu = device_compute_units();
     const int bms[4] = {128, 256, 256, 256}, bns[4] = {128, 128, 192, 256};
-    const double eff[4] = {1.0, 0.92, 1.23, 1.15}; // relative throughput of a busy compute unit, measured on 7B shapes
+    const double eff[4] = {1.0, 1.05, 1.23, 1.15}; // relative throughput of a busy compute unit, measured on 7B shapes
     int best = -1;
     double best_t = 0.0;
     for (int t = 0; t < 4; t++) {
