@@ -13,6 +13,8 @@
 //     tile edge: 128 x 128 moves 1 byte per 64 flop, 256 x 256 one per 128 flop.  launch_gemm_f16_dma picks the
 //     tile by a small cost model (rounds of workgroups over the compute units x tile efficiency).
 // Wavefronts form a (kWavesM x 2) grid; each owns 64 x (32 kNT) of C = 2 x kNT v_mfma_f32_32x32x16_f16 tiles.
+// The same kernel runs on fp32 operands (f32 mode, v_mfma_f32_32x32x2_f32) and, for products with few output tiles,
+// on K ranges whose partial sums gemm_split_finish_kernel adds up (both further down).
 #include "kernels.h"
 #include "device_utils.h"
 
