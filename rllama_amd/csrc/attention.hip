@@ -117,24 +117,35 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
                 vraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(vbase + off) + 16 * w);
             }
         }
+        // the scores of the batch first (independent of each other), then one new maximum and one rescale for the batch:
+        // one exponential per position and one per batch instead of two per position in a serial chain
+        float sc[kAttnBatch];
+        float m_new = m_run;
 #pragma unroll
         for (int u = 0; u < kAttnBatch; u++) {
-            float kc[8], vc[8];
+            float kc[8];
             unpack8<CT>(kraw[u], kc);
-            unpack8<CT>(vraw[u], vc);
             float part = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; i++) part = fmaf(qv[i], kc[i], part);
-            const float s = group_sum<kLanesPerPos>(part) * scale;
-            if (t + u * stride < t1) {
-                const float m_new = fmaxf(m_run, s);
-                const float alpha = expf(m_run - m_new);
-                const float pe = expf(s - m_new);
-                l_run = fmaf(l_run, alpha, pe);
+            sc[u] = t + u * stride < t1 ? group_sum<kLanesPerPos>(part) * scale : -INFINITY;
+            m_new = fmaxf(m_new, sc[u]);
+        }
+        if (m_new > -INFINITY) { // some position of the batch belongs to this lane group (or earlier ones did)
+            const float alpha = expf(m_run - m_new); // first batch: exp(-inf) = 0
+            l_run *= alpha;
 #pragma unroll
-                for (int i = 0; i < 8; i++) acc[i] = fmaf(acc[i], alpha, pe * vc[i]);
-                m_run = m_new;
+            for (int i = 0; i < 8; i++) acc[i] *= alpha;
+#pragma unroll
+            for (int u = 0; u < kAttnBatch; u++) {
+                float vc[8];
+                unpack8<CT>(vraw[u], vc);
+                const float pe = expf(sc[u] - m_new); // positions past the end: exp(-inf) = 0
+                l_run += pe;
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[i] = fmaf(pe, vc[i], acc[i]);
             }
+            m_run = m_new;
         }
     }
 
@@ -147,15 +158,22 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
 #pragma unroll
     for (int i = 0; i < 8; i++) pacc[set][dl * 8 + i] = acc[i];
     __syncthreads();
+    // one weight exp(m_s - M) per lane group, computed once (not once per output dim) and left in pm
+    static_assert(kSets <= kAttnThreads, "one thread per lane group");
+    float M = -INFINITY;
+    for (int s2 = 0; s2 < kSets; s2++) M = fmaxf(M, pm[s2]);
+    float f = 0.0f;
+    if (tid < kSets) f = pl[tid] > 0.0f ? expf(pm[tid] - M) : 0.0f;
+    __syncthreads(); // everybody has read the maxima
+    if (tid < kSets) pm[tid] = f;
+    __syncthreads();
     if (tid < kHeadDim) {
-        float M = -INFINITY;
-        for (int s2 = 0; s2 < kSets; s2++) M = fmaxf(M, pm[s2]);
         float L = 0.0f, O = 0.0f;
+#pragma unroll 8
         for (int s2 = 0; s2 < kSets; s2++) {
-            const float ls = pl[s2];
-            const float f = ls > 0.0f ? expf(pm[s2] - M) : 0.0f;
-            L = fmaf(ls, f, L);
-            O = fmaf(pacc[s2][tid], f, O);
+            const float f2 = pm[s2];
+            L = fmaf(pl[s2], f2, L);
+            O = fmaf(pacc[s2][tid], f2, O);
         }
         if (S == 1) {
             const float o = O / L;
