@@ -117,7 +117,7 @@ struct rlh_model {
     int prompt_cap = 0;
     float *attn_ws = nullptr;
     int max_splits = 32;
-    int attn_single_max = 256; // sequence lengths up to this use one block per head
+    int attn_single_max = 384; // sequence lengths up to this use one block per head (measured: one block 5.6 us at 384 positions against 6.5 us split + merge; 7.1 against 6.4 at 512)
     int attn_chunk = 128;      // positions per block beyond that
     int stream_weights = 1;
     PrefillScratch pf;

@@ -534,25 +534,25 @@ def test_prefill_matrix_core_path_against_token_by_token_and_oracle(ctx):
 def test_decode_step_graph_replay(ctx, monkeypatch):
     """RLLAMA_HIP_DECODE_GRAPH=1 replays the captured decode step (one graph per attention grid shape): the ids are those of
     the eager loop on every replay, across a change of grid shape, with eager work on other caches between the replays."""
-    shape = Shape(dim=256, n_layers=2, n_heads=2, ffn_hidden=512, vocab_size=300, max_seq_len=400)
+    shape = Shape(dim=256, n_layers=2, n_heads=2, ffn_hidden=512, vocab_size=300, max_seq_len=460)
     W = synth_weights(shape, seed=61, std=0.08, norm_ones=False)
     gm = make_gpu(ctx, shape, W, True)
-    prompt = np.random.default_rng(62).integers(0, shape.vocab_size, 248)
+    prompt = np.random.default_rng(62).integers(0, shape.vocab_size, 376)
     monkeypatch.delenv("RLLAMA_HIP_DECODE_GRAPH", raising=False)
     want, _, _ = gm.generate_greedy(prompt, 60, gm.make_caches())
     monkeypatch.setenv("RLLAMA_HIP_DECODE_GRAPH", "1")
     c = gm.make_caches()
-    got, _, _ = gm.generate_greedy(prompt, 20, c)           # positions 248 .. 267: the attention grid changes at 256
+    got, _, _ = gm.generate_greedy(prompt, 20, c)           # positions 376 .. 395: the attention grid changes at 384
     assert np.array_equal(got, want[:20])
     for lo in (20, 40):
         other = gm.make_caches()
         gm.forward(prompt[:17], 0, other)                    # eager work between the replays (it drops the greedy state)
         gm.forward([5], 17, other)
-        # token want[lo - 1] sits at position 248 + lo - 1; forwarding it again yields want[lo] and re-seeds the greedy state
-        assert gm.forward_greedy([int(want[lo - 1])], 248 + lo - 1, c) == want[lo]
+        # token want[lo - 1] sits at position 376 + lo - 1; forwarding it again yields want[lo] and re-seeds the greedy state
+        assert gm.forward_greedy([int(want[lo - 1])], 376 + lo - 1, c) == want[lo]
         if lo == 40:
             c = c.true_clone()                               # a clone replays its own captures, not its source's
-            assert gm.forward_greedy([int(want[lo - 1])], 248 + lo - 1, c) == want[lo]
+            assert gm.forward_greedy([int(want[lo - 1])], 376 + lo - 1, c) == want[lo]
         ids, _ = gm.decode_greedy(19, c)
         assert np.array_equal(ids, want[lo + 1:lo + 20])
     gm.free()
