@@ -31,11 +31,13 @@ typedef __attribute__((ext_vector_type(16))) float float16_t;
 // kF32: the operands are fp32 (f32 mode: tensor.rs:1282-1475 for src.rows > 1).  Staging moves bytes and is the same
 // with a row of kBK / 2 floats; a 16-byte fragment then holds 4 consecutive k of a row and feeds 4
 // v_mfma_f32_32x32x2_f32 (k slot of lane half h in the j-th of them: float j of chunk 2 ks + h, for A and B alike).
-template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false>
+// kIT: 32-row MFMA tiles per wavefront (2: wavefronts of 64 x 32 kNT; 1: 32 x 32 kNT, for products with at most 32 rows).
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false, int kIT = 2>
 __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams p) {
     constexpr int kE = kF32 ? 2 : 1;                     // halves per operand element: k, lda, ldb, strides count elements
     constexpr int kWaves = 2 * kWavesM;
-    constexpr int kBM = 64 * kWavesM, kBN = 64 * kNT;
+    constexpr int kWR = 32 * kIT;                        // rows of a wavefront's tile
+    constexpr int kBM = kWR * kWavesM, kBN = 64 * kNT;
     constexpr int kCpr = kBK / 8;                        // 16-byte chunks per LDS row
     constexpr int kRowsPerLoad = 64 / kCpr;              // rows one wavefront-wide load covers (1 KiB of LDS)
     constexpr int kSwzDiv = 16 / kCpr;                   // physical chunk = logical chunk ^ ((row / kSwzDiv) % kCpr)
@@ -123,9 +125,9 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         }
     };
 
-    float16_t acc[2][kNT];
+    float16_t acc[kIT][kNT];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < kIT; i++)
 #pragma unroll
         for (int j = 0; j < kNT; j++)
 #pragma unroll
@@ -135,16 +137,16 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // latency is gone by the time the accumulators are ready (these ordinary loads are older than every direct-to-LDS
     // load below, so the hand-placed vmcnt waits only get stricter).  Each element is read and later written by the
     // same lane, so C may alias the residual.
-    constexpr bool kEarlyResidual = kEpi == kGemmEpiResAddF32 && kNT <= 2;
-    [[maybe_unused]] float16_t early[kEarlyResidual ? 2 : 1][kEarlyResidual ? kNT : 1];
+    constexpr bool kEarlyResidual = kEpi == kGemmEpiResAddF32 && kNT * kIT <= 4;
+    [[maybe_unused]] float16_t early[kEarlyResidual ? kIT : 1][kEarlyResidual ? kNT : 1];
     if constexpr (kEarlyResidual) {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < kIT; i++)
 #pragma unroll
             for (int j = 0; j < kNT; j++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    const int r = bm0 + wm * 64 + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                    const int r = bm0 + wm * kWR + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
                     const int c = bn0 + wn * (32 * kNT) + j * 32 + (lane & 31);
                     early[i][j][v] = (r < M && c < N) ? p.residual[(size_t)r * p.ldc + c] : 0.0f;
                 }
@@ -154,16 +156,17 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // are fetched now as well, for the same reason.
     [[maybe_unused]] const bool rows16 = (p.ldc % 8) == 0 && (N % 8) == 0 && ((zb * p.stride_c) % 8) == 0 && (reinterpret_cast<uintptr_t>(p.c) % 16) == 0 &&
                                          (kEpi != kGemmEpiSiluGateF16 || (reinterpret_cast<uintptr_t>(p.gate) % 16) == 0);
-    constexpr bool kGatePre = kEpi == kGemmEpiSiluGateF16 && kNT <= 3; // the widest tile has no registers to spare for it
-    constexpr int kGateChunks = kGatePre ? 32 * kNT / 8 : 1;
+    constexpr bool kGatePre = kEpi == kGemmEpiSiluGateF16 && kNT * kIT <= 6; // the widest tile has no registers to spare for it
+    constexpr int kRowChunks = 32 * kNT / 8;             // 16-byte pieces per row of a wavefront's tile
+    constexpr int kGateChunks = kGatePre ? kRowChunks * kWR / 64 : 1;
     [[maybe_unused]] half8_t gate_pre[kGateChunks];
     if constexpr (kGatePre) {
         if (rows16) {
 #pragma unroll
             for (int it = 0; it < kGateChunks; it++) {
                 const int idx = it * 64 + lane;
-                const int rr = idx / kGateChunks, ch = idx - rr * kGateChunks;
-                const int r = bm0 + wm * 64 + rr, c = bn0 + wn * (32 * kNT) + ch * 8;
+                const int rr = idx / kRowChunks, ch = idx - rr * kRowChunks;
+                const int r = bm0 + wm * kWR + rr, c = bn0 + wn * (32 * kNT) + ch * 8;
                 gate_pre[it] = (r < M && c < N) ? *reinterpret_cast<const half8_t *>(p.gate + (size_t)r * p.ldc + c) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
             }
         }
@@ -171,10 +174,10 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 
     // operand fragments: lane l supplies row (l % 32), logical chunk 2 * ks + l / 32 of a 32 x 16 slab
     const int frow = lane & 31, fch = lane >> 5;
-    int a_off[2], a_sw[2], b_off[kNT], b_sw[kNT];
+    int a_off[kIT], a_sw[kIT], b_off[kNT], b_sw[kNT];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int ra = wm * 64 + i * 32 + frow;
+    for (int i = 0; i < kIT; i++) {
+        const int ra = wm * kWR + i * 32 + frow;
         a_off[i] = ra * kRowBytes;
         a_sw[i] = (ra / kSwzDiv) % kCpr;
     }
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     constexpr int kKS = kBK / 16;
     constexpr int kSplitJ = kNT / 2; // column tiles of the last K-step whose MFMAs run before the tile change (0 .. kNT measured alike)
     static_assert(kKS % 2 == 0, "fragment sets alternate by K-step parity");
-    half8_t af[2][2], bf[2][kNT];
+    half8_t af[2][kIT], bf[2][kNT];
     auto mma = [&](const half8_t &a, const half8_t &b, float16_t &c) {
         if constexpr (kF32) {
             const float4_t a4 = __builtin_bit_cast(float4_t, a), b4 = __builtin_bit_cast(float4_t, b);
@@ -206,7 +209,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     auto read_frags = [&](int set, const unsigned char *stage, int ks) {
         const int lc = ks * 2 + fch;
 #pragma unroll
-        for (int i = 0; i < 2; i++) af[set][i] = *reinterpret_cast<const half8_t *>(stage + a_off[i] + ((lc ^ a_sw[i]) << 4));
+        for (int i = 0; i < kIT; i++) af[set][i] = *reinterpret_cast<const half8_t *>(stage + a_off[i] + ((lc ^ a_sw[i]) << 4));
 #pragma unroll
         for (int j = 0; j < kNT; j++) bf[set][j] = *reinterpret_cast<const half8_t *>(stage + b_off[j] + ((lc ^ b_sw[j]) << 4));
     };
@@ -226,12 +229,12 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
                 for (int j = 0; j < kNT; j++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                    for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
                 {   // order within the step: an LDS fragment read of the next step behind each of the first MFMAs of this one,
                     // so that the reads are in flight under the matrix pipe and none is left to wait for when the next step
                     // begins (left to itself the scheduler issues the reads at the end of the step and the MFMAs wait for them)
                     constexpr int kPerMma = kF32 ? 4 : 1; // MFMA instructions per fragment pair
-                    constexpr int kMmas = 2 * kNT, kReads = 2 + kNT, kPairs = kMmas < kReads ? kMmas : kReads;
+                    constexpr int kMmas = kIT * kNT, kReads = kIT + kNT, kPairs = kMmas < kReads ? kMmas : kReads;
 #pragma unroll
                     for (int r = 0; r < kPairs; r++) {
                         __builtin_amdgcn_sched_group_barrier(0x008, kPerMma, 0); // MFMA
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
                 for (int j = 0; j < kSplitJ; j++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                    for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
                 __builtin_amdgcn_sched_barrier(0);
                 if (short_wave) wait_vmcnt<(kStages - 2) * kLoadsMin>();
                 else wait_vmcnt<(kStages - 2) * kLoadsMax>();
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
                 for (int j = kSplitJ; j < kNT; j++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                    for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
             }
         }
     }
@@ -264,7 +267,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // ---- epilogue.  Accumulator register v of a 32 x 32 tile: row 8 * (v / 4) + 4 * (lane / 32) + v % 4, col lane % 32
     const int col_in = lane & 31;
     const int row_in = (lane >> 5) * 4;
-    auto out_row = [&](int i, int v) { return bm0 + wm * 64 + i * 32 + (v >> 2) * 8 + row_in + (v & 3); };
+    auto out_row = [&](int i, int v) { return bm0 + wm * kWR + i * 32 + (v >> 2) * 8 + row_in + (v & 3); };
     auto out_col = [&](int j) { return bn0 + wn * (32 * kNT) + j * 32 + col_in; };
     // f16 outputs whose rows are 16-byte aligned go through LDS (the stages are free now): every wavefront lays its 64 x 32 kNT
     // tile out as rows, then stores whole 16-byte pieces of consecutive columns (and, with the SiLU gate, reads the gate the
@@ -272,14 +275,14 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     if constexpr (kEpi == kGemmEpiF16 || kEpi == kGemmEpiSiluGateF16) {
         if (rows16) { // uniform for the launch
             constexpr int kTW = 32 * kNT; // tile width of a wavefront
-            constexpr int kPad = (kWaves * 64 * (kTW + 8) * 2 <= kStages * kStageBytes) ? 8 : 0;
+            constexpr int kPad = (kWaves * kWR * (kTW + 8) * 2 <= kStages * kStageBytes) ? 8 : 0;
             constexpr int kTS = kTW + kPad; // halves per LDS row
-            static_assert(kWaves * 64 * kTS * 2 <= kStages * kStageBytes, "the output tiles reuse the stages");
+            static_assert(kWaves * kWR * kTS * 2 <= kStages * kStageBytes, "the output tiles reuse the stages");
             constexpr int kChunks = kTW / 8;
             __syncthreads(); // every wavefront has read its last fragments
-            half_t *tile = reinterpret_cast<half_t *>(lds_raw) + wave * (64 * kTS);
+            half_t *tile = reinterpret_cast<half_t *>(lds_raw) + wave * (kWR * kTS);
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < kIT; i++)
 #pragma unroll
                 for (int j = 0; j < kNT; j++)
 #pragma unroll
@@ -287,10 +290,10 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                         tile[(i * 32 + (v >> 2) * 8 + row_in + (v & 3)) * kTS + j * 32 + col_in] = (half_t)acc[i][j][v]; // tensor.rs:1623-1643
             half_t *cbase = reinterpret_cast<half_t *>(p.c) + zb * p.stride_c;
 #pragma unroll
-            for (int it = 0; it < kChunks; it++) {
+            for (int it = 0; it < kChunks * kWR / 64; it++) {
                 const int idx = it * 64 + lane;
                 const int rr = idx / kChunks, ch = idx - rr * kChunks;
-                const int r = bm0 + wm * 64 + rr, c = bn0 + wn * kTW + ch * 8;
+                const int r = bm0 + wm * kWR + rr, c = bn0 + wn * kTW + ch * 8;
                 if (r < M && c < N) {
                     half8_t o = *reinterpret_cast<const half8_t *>(tile + rr * kTS + ch * 8);
                     const size_t off = (size_t)r * p.ldc + c;
@@ -318,13 +321,13 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
     for (int j = 0; j < kNT; j++) {
         const int c = out_col(j);
-        [[maybe_unused]] float16_t prev[2];
+        [[maybe_unused]] float16_t prev[kIT];
         if constexpr (kEarlyResidual) {
-            prev[0] = early[0][j];
-            prev[1] = early[1][j];
+#pragma unroll
+            for (int i = 0; i < kIT; i++) prev[i] = early[i][j];
         } else if constexpr (kEpi == kGemmEpiSiluGateF16) {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < kIT; i++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const int r = out_row(i, v);
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                 }
         } else if constexpr (kEpi != kGemmEpiF16) {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < kIT; i++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const int r = out_row(i, v);
@@ -340,7 +343,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                 }
         }
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < kIT; i++) {
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int r = out_row(i, v);
@@ -371,16 +374,16 @@ bool gemm_f16_dma_supported(const GemmParams &p) {
     return p.causal >= 0 && p.causal <= 2;
 }
 
-template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false>
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false, int kIT = 2>
 static hipError_t launch_dma(const GemmParams &p, hipStream_t s) {
-    constexpr int bm = 64 * kWavesM, bn = 64 * kNT;
+    constexpr int bm = 32 * kIT * kWavesM, bn = 64 * kNT;
     constexpr size_t lds = (size_t)kStages * (bm + bn) * kBK * 2;
     static_assert(lds <= 160 * 1024, "LDS of one compute unit");
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32>),
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32, kIT>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) return attr;
     dim3 grid((p.n + bn - 1) / bn, (p.m + bm - 1) / bm, p.batch);
-    hipLaunchKernelGGL((gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32>), grid, dim3(128 * kWavesM), lds, s, p);
+    hipLaunchKernelGGL((gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32, kIT>), grid, dim3(128 * kWavesM), lds, s, p);
     return hipGetLastError();
 }
 
@@ -405,6 +408,8 @@ static hipError_t launch_dma_epi(const GemmParams &p, int tile, hipStream_t s) {
     case 0: return launch_dma<kEpi, 2, 2, 64, 2>(p, s);  // 128 x 128, 64 KiB of LDS: two workgroups per compute unit
     case 4: return launch_dma<kEpi, 2, 2, 64, 4>(p, s);  // 128 x 128, 128 KiB: one workgroup per compute unit, three K-tiles ahead
     case 5: return launch_dma<kEpi, 2, 1, 64, 6>(p, s);  // 128 x 64, 144 KiB: few rows, so twice the workgroups stream the weights
+    case 6: return launch_dma<kEpi, 1, 1, 64, 10, false, 1>(p, s);  // 32 x 64, 120 KiB: at most 32 rows, nine weight tiles in flight per workgroup
+    case 7: return launch_dma<kEpi, 1, 1, 64, 8, false, 2>(p, s);   // 64 x 64, 128 KiB: at most 64 rows
     case 1: return k64 ? launch_dma<kEpi, 4, 2, 64, 3>(p, s) : launch_dma<kEpi, 4, 2, 32, 4>(p, s);  // 256 x 128
     case 2: return k64 ? launch_dma<kEpi, 4, 3, 64, 2>(p, s) : launch_dma<kEpi, 4, 3, 32, 4>(p, s);  // 256 x 192
     case 3: return k64 ? launch_dma<kEpi, 4, 4, 64, 2>(p, s) : launch_dma<kEpi, 4, 4, 32, 4>(p, s);  // 256 x 256
@@ -549,7 +554,7 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         if (blocks <= device_compute_units()) tile = 4;
         // one row tile and few column tiles (a short prompt): half the tile width, so that twice the workgroups stream the
         // weights; the pieces of a split product use it too
-        if (!p.f32_operands && p.m <= 128 && (p.batch == 1 || p.split_k > 1) && (long)((p.n + 127) / 128) * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = 5;
+        if (!p.f32_operands && p.m <= 128 && (p.batch == 1 || p.split_k > 1) && (long)((p.n + 127) / 128) * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = p.m <= 32 ? 6 : p.m <= 64 ? 7 : 5;
     }
     if (p.f32_operands) {
         if (epilogue != kGemmEpiF32 || ((p.k * 2) % 64) != 0 || (p.k_seg != 0 && ((p.k_seg * 2) % 64) != 0)) return hipErrorInvalidValue;
