@@ -53,7 +53,6 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     int bx = blockIdx.x, by = blockIdx.y;
-#ifndef RLH_GEMM_NO_XCD
     if (gridDim.x % 8 != 0) {
         // Workgroups go to the 8 XCDs round-robin in launch order (x fastest).  With a row of tiles that is not a multiple of
         // 8 wide, the row tiles of one column tile (same B rows) would land on different XCDs and each L2 would fetch that B
@@ -65,7 +64,6 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         by = j / w;
         bx = chunk * 8 + (j - by * w);
     }
-#endif
     const int bm0 = by * kBM, bn0 = bx * kBN;
     const size_t zb = blockIdx.z;
     const half_t *A = p.a + zb * p.stride_a * kE;
