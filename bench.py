@@ -24,9 +24,9 @@ sys.path.insert(0, ROOT)
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per launch of the dominant decode kernel (w13 GEMV, 7B shape) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# HBM bytes per launch of the dominant kernel (c1: w13 GEMV; c3: w1-shape GEMM; 7B shapes) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs, each scaled by the same counter on a 1 GiB copy kernel (the PMC summary under profiles/ has the commands).
-MEASURED_TRAFFIC = {"c1": 181_001_709}
+MEASURED_TRAFFIC = {"c1": 181_001_709, "c3": 186_436_198}
 
 CONFIGS = {
     # name: (dim, n_layers, n_heads, ffn_hidden, vocab, n_prompt, default decode steps)
@@ -176,8 +176,9 @@ def main() -> int:
             "ms_hip_events": round(ev_ms, 3), "tokens_per_s": round(n / (wall_ms * 1e-3), 1),
             "tflops_end_to_end": round(tflops, 1), "algorithmic_flops_end_to_end": flops_linear + flops_attn + flops_head,
             "roofline": {"bound": "mfma", "kernel": f"gemm_f16_dma_kernel (256x192 tile, v_mfma_f32_32x32x16_f16) on the w1/w3 product {n}x{ffn}x{dim}",
-                         "achieved": round(gemm_tflops, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(gemm_tflops / 2500.0, 4), "traffic": None,
-                         "us_per_launch": round(gemm_us, 2), "algorithmic_flops": gemm_flops},
+                         "achieved": round(gemm_tflops, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(gemm_tflops / 2500.0, 4), "traffic": MEASURED_TRAFFIC.get("c3"),
+                         "us_per_launch": round(gemm_us, 2), "algorithmic_flops": gemm_flops,
+                         "algorithmic_bytes_per_launch": 2 * (n * dim + ffn * dim + n * ffn)},
             "cpu_baseline": None, "device": info["name"],
         }
         print(json.dumps(out))
