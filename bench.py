@@ -86,6 +86,56 @@ def cpu_baseline(model, dim, n_layers, n_heads, ffn, vocab, n_prompt=8, n_decode
     }
 
 
+def bench_layer_split(args, ra, ctx, info) -> int:
+    """The device's share of a model split by percentage_to_gpu: one prompt call, then K single-token calls of
+    rlh_forward_layers, each taking the stream from host memory and returning it there (the hand-off the reference makes at
+    the layer boundary).  The host-side blocks are the caller's and are not part of this figure."""
+    dim, n_layers, n_heads, ffn, vocab, n_prompt, dflt_steps = CONFIGS[args.config]
+    K = args.steps if args.steps is not None else dflt_steps
+    W = max(0, args.warmup)
+    max_seq = n_prompt + K + W + 1
+    ds = ra.DataSettings(ctx).force_f16().percentage_to_gpu(args.percentage_to_gpu)
+    model = ra.Transformer(ctx, dim, n_layers, n_heads, ffn, vocab, max_seq, 1e-6, ds)
+    model.fill_synthetic(seed=0, std=0.02)
+    last = model.last_layer_on_gpu()
+    cc = model.make_caches()
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((n_prompt, dim)).astype(np.float32)
+    model.forward_layers(x, 0, cc, 0, last)                                  # sizes the work buffers
+    t0 = time.perf_counter()
+    y = model.forward_layers(x, 0, cc, 0, last)
+    prompt_ms = 1e3 * (time.perf_counter() - t0)
+    row = y[-1:].copy()
+    pos = n_prompt
+    for _ in range(W):
+        row = model.forward_layers(row, pos, cc, 0, last)
+        pos += 1
+    t0 = time.perf_counter()
+    for _ in range(K):
+        row = model.forward_layers(row, pos, cc, 0, last)
+        pos += 1
+    ms = 1e3 * (time.perf_counter() - t0) / K
+    n_res = last + 1
+    t_mean = n_prompt + W + (K + 1) / 2.0
+    bytes_call = n_res * ((4 * dim * dim + 3 * dim * ffn) * 2 + 2 * t_mean * dim * 2 + 2 * dim * 2)
+    out = {
+        "metric": "ms per token, device share of a layer-split LLaMA-7B-shape f16 model (stream handed over per call), 1 MI355X",
+        "value": round(ms, 4), "unit": "ms/token", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16 weights, fp32 accumulate",
+        "data": "synthetic (random-init N(0,0.02) weights seed 0, random stream rows)",
+        "config": {"workload": f"{args.config}: dim {dim}, layers 0..{last} of {n_layers} on the device (percentage_to_gpu {args.percentage_to_gpu}), "
+                               f"{n_prompt}-row prompt call then {K} single-row calls"},
+        "prompt_call_ms": round(prompt_ms, 3), "us_per_resident_layer": round(1e3 * ms / n_res, 2),
+        "handoff_bytes_per_call": 2 * dim * 4,
+        "roofline": {"bound": "hbm", "achieved": round(bytes_call / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(bytes_call / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_call": int(bytes_call)},
+        "cpu_baseline": None, "device": info["name"],
+    }
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -97,6 +147,9 @@ def main() -> int:
     ap.add_argument("--kernels-only", action="store_true",
                     help="skip the token loop and the CPU baseline: only the per-kernel timing loops (short runs for "
                          "rocprofv3 --pmc passes)")
+    ap.add_argument("--percentage-to-gpu", type=float, default=1.0,
+                    help="below 1: time the device's share of a layer-split model (rlh_forward_layers over layers "
+                         "0..=round(p * (n_layers - 1)), stream handed over from and to host memory on every call)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain copy kernel over 1 GiB of f32 (reads 1 GiB, writes 1 GiB per launch): "
                          "the known-size reference for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -127,6 +180,8 @@ def main() -> int:
 
     ctx = ra.Context(0, verbose=False)
     info = ctx.device_info()
+    if args.percentage_to_gpu < 1.0:
+        return bench_layer_split(args, ra, ctx, info)
     ds = ra.DataSettings(ctx).force_f16()
     model = ra.Transformer(ctx, dim, n_layers, n_heads, ffn, vocab, max_seq, 1e-6, ds)
     model.fill_synthetic(seed=0, std=0.02)

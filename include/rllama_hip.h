@@ -91,8 +91,10 @@ typedef struct {
                                    projection weights, f16 KV cache and the f16 rounding points of
                                    src/transformer.rs:665-668, 537-540, 563-565, 795;
                                    0 = f32 weights, f32 KV cache, no rounding anywhere */
-    float   percentage_to_gpu;  /* --percentage-to-gpu; clamped like src/transformer.rs:91-103.  On one
-                                   288 GB device every layer is resident: see rlh_model_layers_on_gpu */
+    float   percentage_to_gpu;  /* --percentage-to-gpu; clamped like src/transformer.rs:91-103.  1.0 (the
+                                   reference's default): every layer is resident.  Below 1.0 only layers
+                                   0..=round(p * (n_layers - 1)) get weights and cache planes on the device
+                                   (src/transformer.rs:262-279): see rlh_forward_layers */
 } rlh_model_params;
 
 int  rlh_model_create(rlh_ctx *ctx, const rlh_model_params *params, rlh_model **out);
@@ -116,7 +118,7 @@ int  rlh_model_fill_synthetic(rlh_model *model, uint64_t seed, double std);
  * Both give the reference's result up to the order of fp32 additions. */
 int  rlh_model_set_prefill_mode(rlh_model *model, int mode);
 /* The layer split rule of src/transformer.rs:262-279: last_layer_on_gpu = round(p * (n_layers - 1)).
- * Reports it; all layers run on the device regardless (nothing is left on the host). */
+ * Layers beyond it have no device storage: rlh_model_set_tensor / get_tensor / rlh_caches_read refuse them. */
 int  rlh_model_layers_on_gpu(const rlh_model *model, int *last_layer_on_gpu);
 /* Bytes of HBM one decode step must read at sequence length T: weights + KV (the roofline's numerator). */
 int  rlh_model_decode_bytes(const rlh_model *model, int T, uint64_t *bytes);
@@ -138,6 +140,17 @@ int  rlh_caches_read(const rlh_caches *caches, int layer, int head, int which, f
  * :350-357 only fits start_pos == 0), start_pos + n <= max_seq_len.  logits_out: vocab floats on the host.
  * ---------------------------------------------------------------------------------------------- */
 int  rlh_forward(rlh_model *model, rlh_caches *caches, const int32_t *tokens, int n, int start_pos, float *logits_out);
+/* The transformer blocks first_layer..=last_layer alone, for a model split by percentage_to_gpu (the loop body of
+ * src/transformer.rs:361-376 over the layers whose DataSettings kept use_opencl, :262-279).  x_in: the n rows of
+ * the residual stream entering first_layer, host f32 [n x dim] (for layer 0 the embedding rows, which the
+ * reference gathers on the host, src/transformer.rs:344-348, src/embedding.rs:41-58).  x_out: the stream
+ * leaving last_layer, same shape (may alias x_in).  The cache planes of those layers are filled at
+ * start_pos..start_pos+n.  Everything else of the forward — the host-side blocks, the final norm and the output
+ * head, which the reference keeps as host tensors (src/transformer.rs:296-308) — stays with the caller's own code:
+ * this library has no host arithmetic.  Same call rules as rlh_forward; also valid on a whole model for any span.
+ * rlh_forward* and the generate loops refuse a split model (RLH_ERR_STATE). */
+int  rlh_forward_layers(rlh_model *model, rlh_caches *caches, const float *x_in, int n, int start_pos, int first_layer, int last_layer,
+                        float *x_out);
 /* forward + TokenSampler::sample with top_k = 1, temperature = 1, repetition_penalty = 1
  * (src/token_sampler.rs:83-174; its loops over 0..logits.rows() only ever touch token 0, whose logit
  * becomes 0.0): the argmax runs on the device, only the id crosses PCIe. */

@@ -95,6 +95,9 @@ def lib() -> C.CDLL:
         "orc_caches_free": (None, [vp]),
         "orc_caches_read": (None, [vp, C.c_int, C.c_int, C.c_int, fp]),
         "orc_forward": (C.c_int, [vp, vp, i32p, C.c_int, C.c_int, fp]),
+        "orc_embed": (C.c_int, [vp, i32p, C.c_int, fp]),
+        "orc_forward_layers": (C.c_int, [vp, vp, fp, C.c_int, C.c_int, C.c_int, C.c_int, fp]),
+        "orc_head": (C.c_int, [vp, fp, C.c_int, fp]),
         "orc_set_layer_tap": (None, [fp]),
     }
     for name, (res, args) in sig.items():
@@ -335,6 +338,31 @@ class Model:
         if rc != 0:
             raise RuntimeError(f"orc_forward -> {rc} (the reference panics here)")
         return (logits, tap) if layer_tap else logits
+
+    # the forward cut at the reference's layer split (transformer.rs:262-279): embed -> forward_layers(...) -> head
+    def embed(self, tokens) -> np.ndarray:
+        toks = np.ascontiguousarray(tokens, dtype=np.int32)
+        x = np.empty((toks.size, self.params.dim), dtype=np.float32)
+        rc = lib().orc_embed(self._h, toks.ctypes.data_as(C.POINTER(C.c_int32)), toks.size, _fp(x))
+        if rc != 0:
+            raise RuntimeError(f"orc_embed -> {rc}")
+        return x
+
+    def forward_layers(self, x: np.ndarray, start_pos: int, caches: Caches, first_layer: int, last_layer: int) -> np.ndarray:
+        xin = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.params.dim)
+        out = np.empty_like(xin)
+        rc = lib().orc_forward_layers(self._h, caches._h, _fp(xin), xin.shape[0], start_pos, first_layer, last_layer, _fp(out))
+        if rc != 0:
+            raise RuntimeError(f"orc_forward_layers -> {rc}")
+        return out
+
+    def head(self, x: np.ndarray) -> np.ndarray:
+        xin = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.params.dim)
+        logits = np.empty(self.params.vocab_size, dtype=np.float32)
+        rc = lib().orc_head(self._h, _fp(xin), xin.shape[0], _fp(logits))
+        if rc != 0:
+            raise RuntimeError(f"orc_head -> {rc}")
+        return logits
 
     def __del__(self):
         if getattr(self, "_h", None):

@@ -731,13 +731,17 @@ static void project(const orc_model *m, const float *x, int n, const void *w, in
     }
 }
 
-int orc_forward(const orc_model *m, orc_caches *c, const int32_t *tokens, int n, int start_pos, float *logits_out) {
+/* Transformer::forward (transformer.rs:343-383) with the places marked where a layer split cuts it: tokens != NULL starts
+ * from the embedding gather, else from the stream x_in; blocks first..=last run; x_out != NULL receives the stream after
+ * them; logits_out != NULL adds the final norm and the head. */
+static int forward_span(const orc_model *m, orc_caches *c, const int32_t *tokens, const float *x_in, int n, int start_pos, int first, int last,
+                        float *x_out, float *logits_out) {
     const orc_params *p = &m->p;
     const int d = p->dim, H = p->n_heads, hd = m->head_dim, F = p->ffn_hidden, V = p->vocab_size;
     if (n < 1) return 1;
     if (n > 1 && start_pos != 0) return 2;      /* mask is n x n, scores are n x (start_pos+n): add panics (tensor.rs:576-584) */
     if (start_pos + n > p->max_seq_len) return 3;
-    for (int i = 0; i < n; i++) {
+    for (int i = 0; tokens && i < n; i++) {
         if (tokens[i] < 0 || tokens[i] >= V) return 4; /* BTreeMap get().unwrap() (embedding.rs:50-52) */
     }
     const int T = start_pos + n;
@@ -755,11 +759,15 @@ int orc_forward(const orc_model *m, orc_caches *c, const int32_t *tokens, int n,
     float *ffn = (float *)malloc(sizeof(float) * (size_t)n * d);
 
     /* embedding gather + concat (transformer.rs:361-367) */
-    for (int i = 0; i < n; i++) memcpy(x + (size_t)i * d, m->tok_emb + (size_t)tokens[i] * d, sizeof(float) * d);
+    if (tokens) {
+        for (int i = 0; i < n; i++) memcpy(x + (size_t)i * d, m->tok_emb + (size_t)tokens[i] * d, sizeof(float) * d);
+    } else {
+        memcpy(x, x_in, sizeof(float) * (size_t)n * d);
+    }
 
     const float inv_sqrt_hd = 1.0f / sqrtf((float)hd); /* transformer.rs:770 */
 
-    for (int l = 0; l < p->n_layers; l++) {
+    for (int l = first; l <= last; l++) {
         const orc_layer *L = &m->layers[l];
         /* attention_norm (transformer.rs:432) */
         for (int i = 0; i < n; i++) orc_rmsnorm_row(x + (size_t)i * d, L->attn_norm, d, p->norm_eps, xn + (size_t)i * d);
@@ -846,10 +854,36 @@ int orc_forward(const orc_model *m, orc_caches *c, const int32_t *tokens, int n,
         for (size_t i = 0; i < (size_t)n * d; i++) x[i] = h[i] + ffn[i];
         if (g_layer_tap) memcpy(g_layer_tap + (size_t)l * n * d, x, sizeof(float) * (size_t)n * d);
     }
-    /* final norm on all rows, last row, output head (transformer.rs:378-381; tensor.rs:1837-1918) */
-    for (int i = 0; i < n; i++) orc_rmsnorm_row(x + (size_t)i * d, m->norm, d, p->norm_eps, xn + (size_t)i * d);
-    matmul_transposed_f32_impl(xn + (size_t)(n - 1) * d, 1, m->output, V, d, logits_out, !g_ref_threading);
+    if (x_out) memcpy(x_out, x, sizeof(float) * (size_t)n * d);
+    if (logits_out) {
+        /* final norm on all rows, last row, output head (transformer.rs:378-381; tensor.rs:1837-1918) */
+        for (int i = 0; i < n; i++) orc_rmsnorm_row(x + (size_t)i * d, m->norm, d, p->norm_eps, xn + (size_t)i * d);
+        matmul_transposed_f32_impl(xn + (size_t)(n - 1) * d, 1, m->output, V, d, logits_out, !g_ref_threading);
+    }
 
     free(x); free(xn); free(q); free(k); free(v); free(att); free(atto); free(h); free(g); free(u); free(ffn);
     return 0;
+}
+
+int orc_forward(const orc_model *m, orc_caches *c, const int32_t *tokens, int n, int start_pos, float *logits_out) {
+    return forward_span(m, c, tokens, NULL, n, start_pos, 0, m->p.n_layers - 1, NULL, logits_out);
+}
+
+int orc_forward_layers(const orc_model *m, orc_caches *c, const float *x_in, int n, int start_pos, int first_layer, int last_layer, float *x_out) {
+    if (first_layer < 0 || last_layer < first_layer || last_layer >= m->p.n_layers) return 5;
+    return forward_span(m, c, NULL, x_in, n, start_pos, first_layer, last_layer, x_out, NULL);
+}
+
+int orc_embed(const orc_model *m, const int32_t *tokens, int n, float *x_out) {
+    for (int i = 0; i < n; i++) {
+        if (tokens[i] < 0 || tokens[i] >= m->p.vocab_size) return 4;
+        memcpy(x_out + (size_t)i * m->p.dim, m->tok_emb + (size_t)tokens[i] * m->p.dim, sizeof(float) * m->p.dim);
+    }
+    return 0;
+}
+
+int orc_head(const orc_model *m, const float *x, int n, float *logits_out) {
+    /* an empty span: no block runs, the stream goes straight to the final norm and the head */
+    if (n < 1) return 1;
+    return forward_span(m, NULL, NULL, x, n, 0, 0, -1, NULL, logits_out);
 }

@@ -138,6 +138,14 @@ void        orc_caches_read(const orc_caches *c, int layer, int head, int which,
  * start_pos + n > max_seq_len). */
 int orc_forward(const orc_model *m, orc_caches *c, const int32_t *tokens, int n, int start_pos, float *logits_out);
 
+/* The same forward cut where the reference's layer split (percentage_to_gpu, transformer.rs:262-279) cuts it, so that a
+ * test can run some blocks elsewhere: orc_embed is the gather of :361-367, orc_forward_layers the blocks
+ * first_layer..=last_layer on a stream x_in [n x dim] (:368-376), orc_head the final norm and output head on the last
+ * row (:378-381).  orc_embed -> orc_forward_layers(0..n_layers-1) -> orc_head is orc_forward bit for bit. */
+int orc_embed(const orc_model *m, const int32_t *tokens, int n, float *x_out);
+int orc_forward_layers(const orc_model *m, orc_caches *c, const float *x_in, int n, int start_pos, int first_layer, int last_layer, float *x_out);
+int orc_head(const orc_model *m, const float *x, int n, float *logits_out);
+
 /* Optional taps for debugging parity: if non-NULL, receives the residual stream [n x dim] after each layer
  * (n_layers * n * dim floats) of the most recent orc_forward call on this thread. */
 void orc_set_layer_tap(float *buf);

@@ -214,6 +214,15 @@ class Transformer:
                                     logits.ctypes.data_as(C.POINTER(C.c_float))))
         return logits
 
+    def forward_layers(self, x: np.ndarray, start_pos: int, caches: TransformerCaches, first_layer: int, last_layer: int) -> np.ndarray:
+        """Blocks first_layer..=last_layer on the n rows of the residual stream x [n x dim] f32 (the loop body of
+        transformer.rs:361-376 for the layers percentage_to_gpu keeps on the device, :262-279). Returns the stream after them."""
+        xin = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.dim)
+        out = np.empty_like(xin)
+        check(self._lib.rlh_forward_layers(self._h, caches._h, xin.ctypes.data_as(C.POINTER(C.c_float)), xin.shape[0], start_pos,
+                                           first_layer, last_layer, out.ctypes.data_as(C.POINTER(C.c_float))))
+        return out
+
     def forward_greedy(self, tokens: Sequence[int], start_pos: int, caches: TransformerCaches) -> int:
         toks = np.ascontiguousarray(tokens, dtype=np.int32)
         nxt = C.c_int32()

@@ -62,6 +62,7 @@ SIGNATURES = {
     "rlh_caches_read": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, _fp]),
     "rlh_forward": (C.c_int, [_vp, _vp, _i32p, C.c_int, C.c_int, _fp]),
     "rlh_forward_greedy": (C.c_int, [_vp, _vp, _i32p, C.c_int, C.c_int, _i32p]),
+    "rlh_forward_layers": (C.c_int, [_vp, _vp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, _fp]),
     "rlh_generate_greedy": (C.c_int, [_vp, _vp, _i32p, C.c_int, C.c_int, _i32p, _fp, _fp]),
     "rlh_decode_greedy": (C.c_int, [_vp, _vp, C.c_int, _i32p, _fp]),
     "rlh_sampler_default": (None, [C.POINTER(SamplerParams)]),

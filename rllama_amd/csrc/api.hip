@@ -103,6 +103,9 @@ struct rlh_model {
     rlh_model_params prm;
     int head_dim = 0;
     int last_layer_on_gpu = 0;
+    // Layers 0 .. n_resident - 1 hold weights and cache planes on the device; with percentage_to_gpu < 1 the rest stay with
+    // the host (transformer.rs:262-279) and only rlh_forward_layers runs on such a model.
+    int n_resident = 0;
     Weight tok_emb, norm, output;
     std::vector<Layer> layers;
     float2 *freqs = nullptr;
@@ -129,6 +132,13 @@ struct rlh_model {
     uint64_t uid = 0;   // unique per created model: a later model at the same address is still another model
     int next_pos = -1;
     rlh_caches *greedy_caches = nullptr;
+};
+
+// A run over some of the layers: the stream enters from and leaves to host memory, no embedding, no output head.
+struct LayerSpan {
+    int first = 0, last = 0;
+    const float *x_in = nullptr; // [n x dim] f32, the stream entering layer `first`
+    float *x_out = nullptr;      // [n x dim] f32, the stream leaving layer `last`
 };
 
 struct rlh_caches {
@@ -287,13 +297,15 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     }
     // transformer.rs:266-268
     m->last_layer_on_gpu = (int)std::round(m->prm.percentage_to_gpu * (float)(prm->n_layers - 1));
+    m->n_resident = m->last_layer_on_gpu + 1;
     m->layers.resize((size_t)prm->n_layers);
     const int d = prm->dim, F = prm->ffn_hidden, V = prm->vocab_size;
     int rc = RLH_OK;
     auto A = [&](Weight &w, int r, int c, int f16) {
         if (rc == RLH_OK) rc = alloc_weight(w, r, c, f16);
     };
-    for (auto &L : m->layers) {
+    for (int l = 0; l < m->n_resident; l++) {
+        Layer &L = m->layers[(size_t)l];
         A(L.wqkv, 3 * d, d, wf16);
         A(L.wo, d, d, wf16);
         A(L.w1, F, d, wf16);
@@ -387,6 +399,10 @@ static int find_slot(rlh_model *m, int kind, int layer, Slot *s) {
     const int d = m->prm.dim, F = m->prm.ffn_hidden, V = m->prm.vocab_size;
     if (kind >= RLH_WQ && kind <= RLH_FFN_NORM) {
         if (layer < 0 || layer >= m->prm.n_layers) return fail(RLH_ERR_INVALID, "layer %d out of range", layer);
+        if (layer >= m->n_resident) {
+            return fail(RLH_ERR_STATE, "layer %d stays on the host: percentage_to_gpu %.4f keeps layers 0..%d on the device (transformer.rs:262-279)",
+                        layer, (double)m->prm.percentage_to_gpu, m->last_layer_on_gpu);
+        }
     }
     Layer *L = (kind >= RLH_WQ && kind <= RLH_FFN_NORM) ? &m->layers[(size_t)layer] : nullptr;
     switch (kind) {
@@ -483,8 +499,9 @@ extern "C" int rlh_model_fill_synthetic(rlh_model *m, uint64_t seed, double std)
     CtxLock lock(m->ctx);
     hipStream_t st = m->ctx->stream;
     const int d = m->prm.dim;
+    const bool whole = m->n_resident == m->prm.n_layers; // a split model leaves embedding, final norm and head to the host (transformer.rs:296-308)
     for (Weight *w : {&m->tok_emb, &m->output}) {
-        if (!w->p) {
+        if (whole && !w->p) {
             int rc = alloc_weight(*w, w->rows, w->cols, 1);
             if (rc != RLH_OK) return rc;
         }
@@ -493,11 +510,14 @@ extern "C" int rlh_model_fill_synthetic(rlh_model *m, uint64_t seed, double std)
         char *dst = (char *)w.p + row_off * (size_t)w.cols * (w.f16 ? 2 : 4);
         return launch_synth_fill(dst, w.f16, (uint64_t)rows * w.cols, synth_key(seed, SYNTH_STREAM_TENSOR(kind, layer)), std, st);
     };
-    HIP_TRY(fill(m->tok_emb, 0, m->tok_emb.rows, RLH_TOK_EMB, 0));
-    HIP_TRY(fill(m->output, 0, m->output.rows, RLH_OUTPUT, 0));
+    if (whole) {
+        HIP_TRY(fill(m->tok_emb, 0, m->tok_emb.rows, RLH_TOK_EMB, 0));
+        HIP_TRY(fill(m->output, 0, m->output.rows, RLH_OUTPUT, 0));
+        m->tok_emb.loaded = m->output.loaded = true;
+    }
     HIP_TRY(launch_fill_f32((float *)m->norm.p, (uint64_t)d, 1.0f, st));
-    m->tok_emb.loaded = m->output.loaded = m->norm.loaded = true;
-    for (int l = 0; l < m->prm.n_layers; l++) {
+    m->norm.loaded = true;
+    for (int l = 0; l < m->n_resident; l++) {
         Layer &L = m->layers[(size_t)l];
         HIP_TRY(fill(L.wqkv, 0, d, RLH_WQ, l));
         HIP_TRY(fill(L.wqkv, (size_t)d, d, RLH_WK, l));
@@ -539,14 +559,19 @@ extern "C" int rlh_model_decode_bytes(const rlh_model *m, int T, uint64_t *bytes
     return RLH_OK;
 }
 
-static int model_ready(const rlh_model *m) {
-    if (!m->tok_emb.loaded || !m->output.loaded || !m->norm.loaded) return 0;
-    for (const auto &L : m->layers) {
+static int layers_ready(const rlh_model *m, int first, int last) {
+    for (int l = first; l <= last; l++) {
+        const Layer &L = m->layers[(size_t)l];
         if (!(L.q_loaded && L.k_loaded && L.v_loaded && L.wo.loaded && L.w1.loaded && L.w2.loaded && L.w3.loaded && L.attn_norm.loaded &&
               L.ffn_norm.loaded))
             return 0;
     }
     return 1;
+}
+
+static int model_ready(const rlh_model *m) {
+    if (!m->tok_emb.loaded || !m->output.loaded || !m->norm.loaded) return 0;
+    return layers_ready(m, 0, m->prm.n_layers - 1);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -560,7 +585,7 @@ extern "C" int rlh_caches_create(rlh_model *m, rlh_caches **out) {
     c->ctx = m->ctx;
     c->model = m;
     c->model_uid = m->uid;
-    c->n_layers = m->prm.n_layers;
+    c->n_layers = m->n_resident; // planes of host-side layers live with the host
     c->n_heads = m->prm.n_heads;
     c->head_dim = m->head_dim;
     c->max_seq_len = m->prm.max_seq_len;
@@ -660,7 +685,7 @@ enum StepKernel { kStepQkv = 0, kStepAttn = 1, kStepWo = 2, kStepW13 = 3, kStepW
 
 // Enqueues one of the five kernels of layer l (or the output head) for the token described by the device
 // state.  T_host = position + 1 as known to the host (sizes the attention grid).
-static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, int T_host) {
+static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, int T_host, int first_layer = 0) {
     hipStream_t st = m->ctx->stream;
     const rlh_model_params &P = m->prm;
     const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size;
@@ -672,7 +697,8 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
     g.x_f16 = f16;
     g.round_y = f16;
     g.eps = eps;
-    // The stream enters layer l in m->x (l == 0: the embedding row) or as m->h + m->ffn_o of layer l - 1.
+    // The stream enters layer l in m->x (l == first_layer: the embedding row, or the row a layer span was handed) or as
+    // m->h + m->ffn_o of layer l - 1.
     if (which == kStepHead) {
         // last residual add + final norm + output head: f32 activations, no rounding
         // (transformer.rs:445, 378-381; tensor.rs:1837-1918)
@@ -703,7 +729,7 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         // write (transformer.rs:432, 665-668, 694-725, 751-761)
         GemvParams p = g;
         p.w = L.wqkv.p;
-        if (l == 0) {
+        if (l == first_layer) {
             p.x = m->x;
         } else {
             p.x = m->h;
@@ -841,7 +867,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
 // Multi-token forward at start_pos == 0 in f16 mode: every projection is one matrix-core GEMM over all n rows
 // (transformer.rs:694-702, 783-815, 551-570 with seq_len > 1), attention is two batched GEMMs per head around a
 // causal softmax (transformer.rs:762-779).  Leaves the last row's logits in m->logits and the KV cache filled.
-static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n) {
+static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, const LayerSpan *span = nullptr) {
     int rc = ensure_prefill_scratch(m, n);
     if (rc != RLH_OK) return rc;
     hipStream_t st = m->ctx->stream;
@@ -850,9 +876,14 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size, H = P.n_heads, hd = m->head_dim;
     const int tp = (n + 63) & ~63; // row stride of this call's scores / probabilities / transposed V (a whole number of K-tiles)
     const float eps = (float)P.norm_eps;
-    HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
-    HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));
-    HIP_TRY(launch_embed_rows(m->tok_emb.p, m->tok_emb.f16, m->prompt_dev, n, d, S.x, st));
+    if (span) {
+        HIP_TRY(hipMemcpyAsync(S.x, span->x_in, sizeof(float) * (size_t)n * d, hipMemcpyHostToDevice, st));
+    } else {
+        HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
+        HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));
+        HIP_TRY(launch_embed_rows(m->tok_emb.p, m->tok_emb.f16, m->prompt_dev, n, d, S.x, st));
+    }
+    const int l_first = span ? span->first : 0, l_last = span ? span->last : P.n_layers - 1;
     const size_t layer_elems = (size_t)H * P.max_seq_len * hd;
     auto gemm = [&](const void *a, int lda, const void *b, int ldb, void *cc, int ldc, int mm, int nn, int kk, int epi, const float *res,
                     const void *gate = nullptr) -> int {
@@ -874,7 +905,7 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         HIP_TRY(launch_gemm_f16(g, epi, st));
         return RLH_OK;
     };
-    for (int l = 0; l < P.n_layers; l++) {
+    for (int l = l_first; l <= l_last; l++) {
         Layer &L = m->layers[(size_t)l];
         char *ck = (char *)c->k + (size_t)l * layer_elems * 2;
         char *cv = (char *)c->v + (size_t)l * layer_elems * 2;
@@ -967,6 +998,10 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         if ((rc = gemm(S.xn, d, L.w3.p, d, S.mm, F, n, F, d, kGemmEpiSiluGateF16, nullptr, S.g)) != RLH_OK) return rc;
         if ((rc = gemm(S.mm, F, L.w2.p, F, S.x, d, n, d, F, kGemmEpiResAddF32, S.h)) != RLH_OK) return rc;    // x = h + w2(...)
     }
+    if (span) {
+        HIP_TRY(hipMemcpyAsync(span->x_out, S.x, sizeof(float) * (size_t)n * d, hipMemcpyDeviceToHost, st));
+        return RLH_OK;
+    }
     // final norm + output head on the last row only (transformer.rs:378-381)
     GemvParams p{};
     p.stream_weights = m->stream_weights;
@@ -989,7 +1024,7 @@ static bool prefill_f32_supported(const rlh_model *m) {
 
 // Multi-token forward at start_pos == 0 in f32 mode: the same structure as enqueue_prefill on fp32 operands
 // (v_mfma_f32_32x32x2_f32), no rounding points, residual adds as accumulating GEMM epilogues on x in place.
-static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n) {
+static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, const LayerSpan *span = nullptr) {
     int rc = ensure_prefill_scratch(m, n);
     if (rc != RLH_OK) return rc;
     hipStream_t st = m->ctx->stream;
@@ -998,9 +1033,14 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
     const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size, H = P.n_heads, hd = m->head_dim;
     const int tp = (n + 63) & ~63;
     const float eps = (float)P.norm_eps;
-    HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
-    HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));
-    HIP_TRY(launch_embed_rows(m->tok_emb.p, m->tok_emb.f16, m->prompt_dev, n, d, S.x, st));
+    if (span) {
+        HIP_TRY(hipMemcpyAsync(S.x, span->x_in, sizeof(float) * (size_t)n * d, hipMemcpyHostToDevice, st));
+    } else {
+        HIP_TRY(hipMemcpyAsync(m->prompt_dev, tokens, sizeof(int32_t) * (size_t)n, hipMemcpyHostToDevice, st));
+        HIP_TRY(launch_set_state(m->state, n - 1, tokens[n - 1], 1, st));
+        HIP_TRY(launch_embed_rows(m->tok_emb.p, m->tok_emb.f16, m->prompt_dev, n, d, S.x, st));
+    }
+    const int l_first = span ? span->first : 0, l_last = span ? span->last : P.n_layers - 1;
     const size_t layer_elems = (size_t)H * P.max_seq_len * hd;
     auto gemm = [&](const void *a, int lda, const void *b, int ldb, float *cc, int ldc, int mm, int nn, int kk, int accumulate) -> int {
         GemmParams g{};
@@ -1021,7 +1061,7 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
     };
     float *xn = (float *)S.xn, *qkv = (float *)S.qkv, *q = (float *)S.q2, *v_t = (float *)S.v_t, *att = (float *)S.a;
     float *gg = (float *)S.g, *uu = (float *)S.u, *mm = (float *)S.mm;
-    for (int l = 0; l < P.n_layers; l++) {
+    for (int l = l_first; l <= l_last; l++) {
         Layer &L = m->layers[(size_t)l];
         float *ck = (float *)c->k + (size_t)l * layer_elems;
         float *cv = (float *)c->v + (size_t)l * layer_elems;
@@ -1086,6 +1126,10 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
         HIP_TRY(launch_silu_mul_f32(gg, uu, mm, (size_t)n * F, st));
         if ((rc = gemm(mm, F, L.w2.p, F, S.x, d, n, d, F, 1)) != RLH_OK) return rc;      // x += w2(...)   (transformer.rs:445)
     }
+    if (span) {
+        HIP_TRY(hipMemcpyAsync(span->x_out, S.x, sizeof(float) * (size_t)n * d, hipMemcpyDeviceToHost, st));
+        return RLH_OK;
+    }
     // final norm + output head on the last row only (transformer.rs:378-381)
     GemvParams p{};
     p.stream_weights = m->stream_weights;
@@ -1104,6 +1148,12 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
 static int check_forward_args(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, const char *who) {
     if (!m || !c || !tokens) return fail(RLH_ERR_INVALID, "%s: NULL argument", who);
     if (c->model != m || c->model_uid != m->uid) return fail(RLH_ERR_STATE, "%s: caches belong to another model", who);
+    if (m->n_resident < m->prm.n_layers) {
+        return fail(RLH_ERR_STATE,
+                    "%s: percentage_to_gpu %.4f keeps layers %d.. on the host (transformer.rs:262-279): run rlh_forward_layers over 0..%d and the "
+                    "remaining blocks, the final norm and the output head with the host's own path",
+                    who, (double)m->prm.percentage_to_gpu, m->n_resident, m->last_layer_on_gpu);
+    }
     if (!model_ready(m)) return fail(RLH_ERR_STATE, "%s: model has tensors that were never set", who);
     if (n < 1) return fail(RLH_ERR_INVALID, "%s: n must be >= 1", who);
     if (n > 1 && start_pos != 0) {
@@ -1162,6 +1212,58 @@ extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *to
     HIP_TRY(hipStreamSynchronize(st));
     m->next_pos = start_pos + n;
     m->greedy_caches = c;
+    return RLH_OK;
+}
+
+extern "C" int rlh_forward_layers(rlh_model *m, rlh_caches *c, const float *x_in, int n, int start_pos, int first_layer, int last_layer,
+                                  float *x_out) {
+    if (!m || !c || !x_in || !x_out) return fail(RLH_ERR_INVALID, "rlh_forward_layers: NULL argument");
+    if (c->model != m || c->model_uid != m->uid) return fail(RLH_ERR_STATE, "rlh_forward_layers: caches belong to another model");
+    if (first_layer < 0 || last_layer < first_layer || last_layer >= m->prm.n_layers) {
+        return fail(RLH_ERR_INVALID, "rlh_forward_layers: layers %d..%d out of range (model has %d)", first_layer, last_layer, m->prm.n_layers);
+    }
+    if (last_layer >= m->n_resident) {
+        return fail(RLH_ERR_STATE, "rlh_forward_layers: layer %d stays on the host: percentage_to_gpu %.4f keeps layers 0..%d on the device",
+                    last_layer, (double)m->prm.percentage_to_gpu, m->last_layer_on_gpu);
+    }
+    if (!layers_ready(m, first_layer, last_layer)) return fail(RLH_ERR_STATE, "rlh_forward_layers: layers %d..%d have tensors that were never set", first_layer, last_layer);
+    if (n < 1) return fail(RLH_ERR_INVALID, "rlh_forward_layers: n must be >= 1");
+    if (n > 1 && start_pos != 0) {
+        return fail(RLH_ERR_INVALID, "rlh_forward_layers: n > 1 needs start_pos == 0 (the reference's mask is n x n, transformer.rs:350-357)");
+    }
+    if (start_pos < 0 || start_pos + n > m->prm.max_seq_len) {
+        return fail(RLH_ERR_STATE, "rlh_forward_layers: start_pos + n = %d exceeds max_seq_len %d", start_pos + n, m->prm.max_seq_len);
+    }
+    CtxLock lock(m->ctx);
+    hipStream_t st = m->ctx->stream;
+    m->next_pos = -1; // the device state no longer describes a sampled token
+    m->greedy_caches = nullptr;
+    LayerSpan span;
+    span.first = first_layer;
+    span.last = last_layer;
+    span.x_in = x_in;
+    span.x_out = x_out;
+    int rc = RLH_OK;
+    if (n > 1 && m->prefill_mode == 0 && (m->prm.force_f16 || prefill_f32_supported(m))) {
+        rc = m->prm.force_f16 ? enqueue_prefill(m, c, nullptr, n, &span) : enqueue_prefill_f32(m, c, nullptr, n, &span);
+        if (rc != RLH_OK) return rc;
+    } else {
+        const int d = m->prm.dim;
+        for (int i = 0; i < n; i++) {
+            HIP_TRY(launch_set_state(m->state, start_pos + i, 0, 1, st));
+            HIP_TRY(hipMemcpyAsync(m->x, x_in + (size_t)i * d, sizeof(float) * (size_t)d, hipMemcpyHostToDevice, st));
+            for (int l = first_layer; l <= last_layer; l++) {
+                for (int which = kStepQkv; which <= kStepW2; which++) {
+                    rc = enqueue_step_kernel(m, c, l, which, start_pos + i + 1, first_layer);
+                    if (rc != RLH_OK) return rc;
+                }
+            }
+            // the last block's second residual add (transformer.rs:445), which a following kernel's prologue would have done
+            HIP_TRY(launch_add_f32(m->x, m->h, m->ffn_o, (uint64_t)d, st));
+            HIP_TRY(hipMemcpyAsync(x_out + (size_t)i * d, m->x, sizeof(float) * (size_t)d, hipMemcpyDeviceToHost, st));
+        }
+    }
+    HIP_TRY(hipStreamSynchronize(st));
     return RLH_OK;
 }
 

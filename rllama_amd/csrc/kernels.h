@@ -173,6 +173,7 @@ hipError_t launch_convert(void *dst, int dst_f16, const void *src, int src_f16, 
 hipError_t launch_transpose(void *dst, const void *src, int rows, int cols, int is_f16, hipStream_t s); // src [rows x cols]
 hipError_t launch_hadamard(void *dst, const void *src, uint64_t n, int is_f16, hipStream_t s);
 hipError_t launch_silu(void *dst, uint64_t n, int is_f16, hipStream_t s);
+hipError_t launch_add_f32(float *dst, const float *a, const float *b, uint64_t n, hipStream_t s); // dst = a + b
 hipError_t launch_rmsnorm_rows(float *y, const float *x, const float *w, int rows, int d, float eps, int round_y, hipStream_t s);
 hipError_t launch_rope_row(float *x, int n_heads, int head_dim, const float2 *freqs_at_pos, hipStream_t s);
 // KV-cache services (transformer.rs:180-197): shift positions left by `shifts` within each (head) plane

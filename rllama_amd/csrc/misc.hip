@@ -247,6 +247,18 @@ hipError_t launch_hadamard(void *dst, const void *src, uint64_t n, int is_f16, h
     return hipGetLastError();
 }
 
+// dst = a + b (Tensor::add, tensor.rs:573-593), f32
+__global__ void add_f32_kernel(float *dst, const float *a, const float *b, uint64_t n) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = a[i] + b[i];
+}
+
+hipError_t launch_add_f32(float *dst, const float *a, const float *b, uint64_t n, hipStream_t s) {
+    dim3 g(fill_blocks(n)), blk(256);
+    hipLaunchKernelGGL(add_f32_kernel, g, blk, 0, s, dst, a, b, n);
+    return hipGetLastError();
+}
+
 template <typename T>
 __global__ void silu_kernel(T *dst, uint64_t n) {
     const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;

@@ -160,6 +160,14 @@ class Transformer {
                                  (int)existing_tokens.size(), u, &tok, &prob));
         return {tok, prob};
     }
+    // The blocks first_layer..=last_layer on the rows of the residual stream x [n x dim] (the loop body of src/transformer.rs:361-376
+    // for the layers percentage_to_gpu keeps on the device, :262-279); the host-side blocks, norm and head are the caller's.
+    std::vector<float> forward_layers(const std::vector<float> &x, size_t n, size_t start_pos, TransformerCaches &caches, int first_layer,
+                                      int last_layer) const {
+        std::vector<float> out(x.size());
+        check(rlh_forward_layers(h_, caches.raw(), x.data(), (int)n, (int)start_pos, first_layer, last_layer, out.data()));
+        return out;
+    }
     int last_layer_on_gpu() const { // src/transformer.rs:266-268
         int v = 0;
         check(rlh_model_layers_on_gpu(h_, &v));

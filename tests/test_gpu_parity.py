@@ -9,7 +9,7 @@ import pytest
 import oracle
 import rllama_amd
 from rllama_amd import Tensor, TensorDType
-from common import (CONFIG0, SMALL, TINY, Shape, make_gpu, make_oracle, max_rel_err, random_f32_weights, synth_weights)
+from common import (CONFIG0, PER_LAYER, SMALL, TINY, Shape, make_gpu, make_oracle, max_rel_err, random_f32_weights, synth_weights)
 
 pytestmark = pytest.mark.gpu
 f32 = np.float32
@@ -438,6 +438,102 @@ def test_percentage_to_gpu_rule(ctx):
                                    shape.max_seq_len, shape.norm_eps, ds)
         assert m.last_layer_on_gpu() == want, p
         m.free()
+
+
+def _make_split_gpu(ctx, shape, W, force_f16, p):
+    ds = rllama_amd.DataSettings(ctx).percentage_to_gpu(p)
+    if force_f16:
+        ds = ds.force_f16()
+    m = rllama_amd.Transformer(ctx, shape.dim, shape.n_layers, shape.n_heads, shape.ffn_hidden, shape.vocab_size, shape.max_seq_len,
+                               shape.norm_eps, ds)
+    last = m.last_layer_on_gpu()
+    for (kind, layer), arr in W.items():
+        if kind in PER_LAYER or kind in (rllama_amd.ATTN_NORM, rllama_amd.FFN_NORM):
+            if layer <= last:
+                m.set_tensor(kind, layer, arr)
+    return m, last
+
+
+@pytest.mark.parametrize("force_f16,token_by_token", [(True, False), (True, True), (False, False), (False, True)],
+                         ids=["f16-matrix-core", "f16-token-by-token", "f32-matrix-core", "f32-token-by-token"])
+def test_hybrid_layer_split(ctx, force_f16, token_by_token):
+    """--percentage-to-gpu (transformer.rs:262-279): blocks 0..=last_layer_on_gpu through rlh_forward_layers, the remaining
+    blocks, the final norm and the head on the host (here the oracle stands in for the reference's own CPU path).  The stream
+    handed over, the device's cache planes and the final logits are compared with the all-host forward, for a prompt call and
+    for single-token calls after it."""
+    shape = SMALL
+    tol = TOL_F16 if force_f16 else TOL_F32
+    W = synth_weights(shape, seed=9, std=0.05, norm_ones=False)
+    om = make_oracle(shape, W, force_f16)
+    toks = [int(t) for t in np.random.default_rng(11).integers(3, shape.vocab_size, 9)]
+    follow = [17, 4, 300]
+    for p in (0.0, 0.5):
+        gm, last = _make_split_gpu(ctx, shape, W, force_f16, p)
+        assert last == round(p * (shape.n_layers - 1)) and last < shape.n_layers - 1
+        gm.set_prefill_mode(token_by_token)
+        gc = gm.make_caches()
+        oc_full, oc_tail = om.make_caches(), om.make_caches()
+        calls = [(toks, 0)] + [([t], len(toks) + i) for i, t in enumerate(follow)]
+        for call_toks, start in calls:
+            want, tap = om.forward(call_toks, start, oc_full, layer_tap=True)
+            x = gm.forward_layers(om.embed(call_toks), start, gc, 0, last)
+            assert max_rel_err(x, tap[last]) < tol, (p, start, max_rel_err(x, tap[last]))
+            y = om.forward_layers(x, start, oc_tail, last + 1, shape.n_layers - 1)
+            got = om.head(y)
+            assert max_rel_err(got, want) < tol, (p, start, max_rel_err(got, want))
+        T = len(toks) + len(follow)
+        for l in range(last + 1):
+            for which in (0, 1):
+                a, b = gc.read(l, 1, which), oc_full.read(l, 1, which)
+                assert max_rel_err(a[:, :T], b[:, :T]) < tol
+                assert not a[:, T:].any()
+        # what a split model refuses: whole forwards, tensors and cache planes of host-side layers
+        with pytest.raises(rllama_amd.RllamaHipError, match="percentage_to_gpu"):
+            gm.forward(toks, 0, gc)
+        with pytest.raises(rllama_amd.RllamaHipError, match="percentage_to_gpu"):
+            gm.generate_greedy(toks, 2, gc)
+        with pytest.raises(rllama_amd.RllamaHipError, match="stays on the host"):
+            gm.set_tensor(rllama_amd.WO, last + 1, W[(rllama_amd.WO, last + 1)])
+        with pytest.raises(rllama_amd.RllamaHipError, match="stays on the host"):
+            gm.forward_layers(om.embed(toks), 0, gc, 0, last + 1)
+        with pytest.raises(rllama_amd.RllamaHipError):
+            gc.read(last + 1, 0, 0)
+        with pytest.raises(rllama_amd.RllamaHipError):
+            gm.forward_layers(om.embed(toks), 1, gc, 0, last)       # n > 1 needs start_pos == 0
+        gc.free()
+        gm.free()
+
+
+def test_layer_span_on_a_whole_model_equals_its_forward(ctx):
+    """On a fully resident model any span runs: two spans back to back give the stream whose norm + head are the logits
+    of rlh_forward, and a span over layers that were never set is refused."""
+    shape = SMALL
+    W = synth_weights(shape, seed=2, std=0.05, norm_ones=False)
+    om = make_oracle(shape, W, True)
+    gm = make_gpu(ctx, shape, W, True)
+    toks = [int(t) for t in np.random.default_rng(5).integers(3, shape.vocab_size, 33)]
+    c1, c2 = gm.make_caches(), gm.make_caches()
+    want = gm.forward(toks, 0, c1)
+    x = gm.forward_layers(om.embed(toks), 0, c2, 0, 0)
+    x = gm.forward_layers(x, 0, c2, 1, shape.n_layers - 1)
+    got = om.head(x)                                   # final norm + f32 head: the host's part in the reference
+    assert max_rel_err(got, want) < 1e-5, max_rel_err(got, want)
+    for l in range(shape.n_layers):
+        assert np.array_equal(c1.read(l, 0, 0), c2.read(l, 0, 0)) and np.array_equal(c1.read(l, 3, 1), c2.read(l, 3, 1))
+    # the caches of a span call continue under the whole forward
+    a = gm.forward([9], len(toks), c1)
+    b = gm.forward([9], len(toks), c2)
+    assert np.array_equal(a, b)
+    empty = rllama_amd.Transformer(ctx, shape.dim, shape.n_layers, shape.n_heads, shape.ffn_hidden, shape.vocab_size, shape.max_seq_len,
+                                   shape.norm_eps, rllama_amd.DataSettings(ctx).force_f16())
+    ce = empty.make_caches()
+    with pytest.raises(rllama_amd.RllamaHipError, match="never set"):
+        empty.forward_layers(om.embed(toks), 0, ce, 0, 0)
+    ce.free()
+    empty.free()
+    c1.free()
+    c2.free()
+    gm.free()
 
 
 # the last four are sized so that the tile choice lands on the 256 x 192, 256 x 256 and 256 x 128 tiles (with ragged edges)

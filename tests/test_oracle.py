@@ -13,6 +13,7 @@ import pytest
 import scipy.special
 
 import oracle
+from rllama_amd import TOK_EMB
 from common import (SMALL, TINY, RefF64, make_oracle, max_rel_err, random_f32_weights, synth_weights)
 
 f32 = np.float32
@@ -405,6 +406,34 @@ def test_forward_with_zeroed_wo_and_w2_is_head_of_normed_embedding():
     xn = e / np.sqrt(np.mean(e * e) + shape.norm_eps) * W[(NORM, 0)][0]
     want = W[(OUTPUT, 0)].view(np.float16).astype(np.float64) @ xn
     assert max_rel_err(got, want) < 1e-5
+
+
+@pytest.mark.parametrize("force_f16", [False, True], ids=["f32", "f16"])
+def test_forward_cut_at_the_layer_split_is_the_same_forward(force_f16):
+    """embed -> forward_layers(0..k) -> forward_layers(k+1..L-1) -> head is forward bit for bit, for a prompt call and a
+    single-token call, at every cut k (the pieces a layer split hands between devices, transformer.rs:262-279, 361-381)."""
+    shape = SMALL
+    W = synth_weights(shape, seed=5, std=0.05, norm_ones=False)
+    m = make_oracle(shape, W, force_f16)
+    toks = [int(t) for t in np.random.default_rng(3).integers(3, shape.vocab_size, 6)]
+    c0 = m.make_caches()
+    want_prompt, tap = m.forward(toks, 0, c0, layer_tap=True)
+    want_next = m.forward([7], len(toks), c0)
+    emb = W[(TOK_EMB, 0)].view(np.float16).astype(np.float32)
+    assert np.array_equal(m.embed(toks), emb[toks])
+    for k in range(shape.n_layers):
+        c = m.make_caches()
+        x = m.forward_layers(m.embed(toks), 0, c, 0, k)
+        assert np.array_equal(x, tap[k]), k
+        if k + 1 < shape.n_layers:
+            x = m.forward_layers(x, 0, c, k + 1, shape.n_layers - 1)
+        assert np.array_equal(m.head(x), want_prompt), k
+        y = m.forward_layers(m.embed([7]), len(toks), c, 0, k)
+        if k + 1 < shape.n_layers:
+            y = m.forward_layers(y, len(toks), c, k + 1, shape.n_layers - 1)
+        assert np.array_equal(m.head(y), want_next), k
+        for l in range(shape.n_layers):
+            assert np.array_equal(c.read(l, 1, 0), c0.read(l, 1, 0)) and np.array_equal(c.read(l, 2, 1), c0.read(l, 2, 1))
 
 
 def test_cache_shift_left():
