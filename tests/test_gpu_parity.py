@@ -690,6 +690,45 @@ def test_full_size_7b_properties(ctx, n_prompt):
     m.free()
 
 
+def test_full_size_7b_layer_split(ctx):
+    """7B shape split by percentage_to_gpu 0.5 (17 of 32 layers resident): its span calls give bit for bit the stream the same
+    span gives on a whole model with the same weights (a prompt call and single-token calls); on the whole model two spans
+    back to back, then the final norm and the head in numpy, give the logits of rlh_forward."""
+    dim, L, H, F, V, n_prompt = 4096, 32, 32, 11008, 32000, 72
+    whole = rllama_amd.Transformer(ctx, dim, L, H, F, V, n_prompt + 8, 1e-6, rllama_amd.DataSettings(ctx).force_f16())
+    whole.fill_synthetic(0, 0.02)
+    split = rllama_amd.Transformer(ctx, dim, L, H, F, V, n_prompt + 8, 1e-6, rllama_amd.DataSettings(ctx).force_f16().percentage_to_gpu(0.5))
+    split.fill_synthetic(0, 0.02)
+    last = split.last_layer_on_gpu()
+    assert last == 16
+    prompt = rllama_amd.synth_tokens(0, n_prompt, 3, V)
+    emb = whole.get_tensor(rllama_amd.TOK_EMB, 0, V, dim)
+    cw, cs, cf = whole.make_caches(), split.make_caches(), whole.make_caches()
+    x = emb[prompt]
+    xs = split.forward_layers(x, 0, cs, 0, last)
+    xw = whole.forward_layers(x, 0, cw, 0, last)
+    assert np.array_equal(xs, xw)
+    xw = whole.forward_layers(xw, 0, cw, last + 1, L - 1)
+    want = whole.forward(prompt, 0, cf)
+
+    def head(row):
+        row = row.astype(np.float64)
+        xn = (row / np.sqrt(np.mean(row * row) + 1e-6)).astype(np.float32)          # final norm, weights 1.0
+        return whole.get_tensor(rllama_amd.OUTPUT, 0, V, dim) @ xn
+
+    assert max_rel_err(head(xw[-1]), want) < 1e-4
+    for step, tok in enumerate((11, 12345)):
+        r = emb[[tok]]
+        rs = split.forward_layers(r, n_prompt + step, cs, 0, last)
+        rw = whole.forward_layers(r, n_prompt + step, cw, 0, last)
+        assert np.array_equal(rs, rw)
+        rw = whole.forward_layers(rw, n_prompt + step, cw, last + 1, L - 1)
+        assert max_rel_err(head(rw[0]), whole.forward([tok], n_prompt + step, cf)) < 1e-4
+    assert np.array_equal(cs.read(last, 7, 1), cw.read(last, 7, 1))
+    split.free()
+    whole.free()
+
+
 @pytest.mark.parametrize("dim,L,H,F,n_prompt", [(5120, 40, 40, 13824, 300), (8192, 80, 64, 22016, 96)], ids=["13B-shape", "65B-shape"])
 def test_full_size_larger_shapes_prefill_equals_token_by_token(ctx, dim, L, H, F, n_prompt):
     """The 13B and 65B shapes of the other configurations (other GEMM tile choices, split factors and attention grids than 7B):
