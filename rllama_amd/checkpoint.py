@@ -331,8 +331,8 @@ _LAYER = {"wq": ("layers.{}.attention.wq.weight", FROM_PIECES_ROWS, False), "wk"
 
 def load_transformer(ctx, model_path: str, data_settings, max_seq_len: int):
     """main's model construction (src/rllama_main.rs:235-283) + Transformer::from_unpickled (src/transformer.rs:242-326):
-    reads every tensor of the directory and hands its f16 bits to the device model (the values the reference gets
-    after its f16 -> f32 -> f16 round trip are the same bits)."""
+    reads every tensor of the directory that belongs on the device and hands its f16 bits to the device model (the values
+    the reference gets after its f16 -> f32 -> f16 round trip are the same bits)."""
     import rllama_amd as ra
 
     ck = Checkpoint(model_path)
@@ -341,9 +341,14 @@ def load_transformer(ctx, model_path: str, data_settings, max_seq_len: int):
     tr = ra.Transformer(ctx, ck.dim, ck.n_layers, ck.n_heads, ffn, ck.vocab_size, max_seq_len, ck.norm_eps, data_settings)
     kinds = {"tok_embeddings": ra.TOK_EMB, "norm": ra.NORM, "output": ra.OUTPUT, "wq": ra.WQ, "wk": ra.WK, "wv": ra.WV, "wo": ra.WO,
              "w1": ra.W1, "w2": ra.W2, "w3": ra.W3, "attention_norm": ra.ATTN_NORM, "ffn_norm": ra.FFN_NORM}
+    # With percentage_to_gpu below 1 only the leading layers live on the device (src/transformer.rs:262-279); the other
+    # blocks, the embedding table and the output head are the host's (it reads them with Checkpoint.load_f16_bits itself).
+    last = tr.last_layer_on_gpu()
+    whole = last == ck.n_layers - 1
     for key, (name, direction, first) in _TOP.items():
-        tr.set_tensor(kinds[key], 0, ck.load_f16_bits(name, direction, first))
-    for l in range(ck.n_layers):
+        if whole or key == "norm":
+            tr.set_tensor(kinds[key], 0, ck.load_f16_bits(name, direction, first))
+    for l in range(last + 1):
         for key, (fmt, direction, first) in _LAYER.items():
             tr.set_tensor(kinds[key], l, ck.load_f16_bits(fmt.format(l), direction, first))
     return tr

@@ -446,8 +446,8 @@ inline HalfMatrix load_from_pieces(const DataSource &src, const std::string &nam
     return m;
 }
 
-// Model construction (src/rllama_main.rs:235-283, src/transformer.rs:242-326): every tensor of the directory goes to the
-// device model.  The FFN width comes from the stored shape of w1 (no params.json field).
+// Model construction (src/rllama_main.rs:235-283, src/transformer.rs:242-326): every tensor of the directory that belongs on
+// the device goes to the device model.  The FFN width comes from the stored shape of w1 (no params.json field).
 inline std::unique_ptr<Transformer> load_transformer(const std::string &model_path, size_t max_seq_len, const DataSettings &data_settings,
                                                      ModelParams *params_out = nullptr) {
     const DataSource src = DataSource::from_inferred_source(model_path);
@@ -460,10 +460,14 @@ inline std::unique_ptr<Transformer> load_transformer(const std::string &model_pa
         const HalfMatrix m = load_from_pieces(src, name, dir, first);
         tr->set_tensor(kind, layer, m.bits.data(), (int)m.rows, (int)m.cols, TensorDType::Float16);
     };
-    put(RLH_TOK_EMB, 0, "tok_embeddings.weight", D::Cols, false); // src/embedding.rs:18-37
-    put(RLH_NORM, 0, "norm.weight", D::Rows, true);               // src/transformer.rs:297-298, 456-467
-    put(RLH_OUTPUT, 0, "output.weight", D::Rows, false);          // :303-308
-    for (size_t l = 0; l < mp.n_layers; l++) {
+    // With percentage_to_gpu below 1 only the leading layers live on the device (src/transformer.rs:262-279); the other
+    // blocks, the embedding table and the output head are the host's, which reads them with load_from_pieces itself.
+    const size_t n_device_layers = (size_t)tr->last_layer_on_gpu() + 1;
+    const bool whole = n_device_layers == mp.n_layers;
+    if (whole) put(RLH_TOK_EMB, 0, "tok_embeddings.weight", D::Cols, false); // src/embedding.rs:18-37
+    put(RLH_NORM, 0, "norm.weight", D::Rows, true);                          // src/transformer.rs:297-298, 456-467
+    if (whole) put(RLH_OUTPUT, 0, "output.weight", D::Rows, false);          // :303-308
+    for (size_t l = 0; l < n_device_layers; l++) {
         const std::string p = "layers." + std::to_string(l) + ".";
         put(RLH_WQ, (int)l, p + "attention.wq.weight", D::Rows, false); // :595-614
         put(RLH_WK, (int)l, p + "attention.wk.weight", D::Rows, false);

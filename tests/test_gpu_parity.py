@@ -792,6 +792,13 @@ def test_model_loaded_from_checkpoint_directory(ctx, tmp_path, shards):
     b = direct.forward(prompt, 0, direct.make_caches())
     assert np.array_equal(a, b)
     want_ids, _, _ = direct.generate_greedy(prompt, n_new, direct.make_caches())
+    # the same directory under a layer split: only the device's layers are loaded, and they run as a span
+    part = checkpoint.load_transformer(ctx, path, rllama_amd.DataSettings(ctx).force_f16().percentage_to_gpu(0.5), shape.max_seq_len)
+    last = part.last_layer_on_gpu()
+    assert last == 1 and shape.n_layers == 3
+    x = W16[(rllama_amd.TOK_EMB, 0)].view(np.float16).astype(np.float32)[prompt]
+    assert np.array_equal(part.forward_layers(x, 0, part.make_caches(), 0, last), direct.forward_layers(x, 0, direct.make_caches(), 0, last))
+    part.free()
     loaded.free()
     direct.free()
     r = subprocess.run([build.build_host(), "--model-path", path, str(n_prompt), str(n_new), "0"], capture_output=True, text=True, timeout=120)
