@@ -12,7 +12,10 @@
  *     src/tensor_opencl_support.rs:77-83, play this role);
  *   - handles are opaque; a handle belongs to the context that made it;
  *   - all calls on one context are serialised by the library (the reference serialises on a
- *     `programs.write()` lock and one in-order queue, src/tensor_opencl_support.rs:120, :322);
+ *     `programs.write()` lock and one in-order queue, src/tensor_opencl_support.rs:120, :322), so
+ *     handles may be shared between threads (DataSettings is Send + Sync, src/transformer.rs:52-53).
+ *     One piece of state is per model, not per call: the sampled id that rlh_decode_greedy continues
+ *     from, so a greedy call on other caches in between (from any thread) makes it refuse;
  *   - host pointers are only read/written during the call unless stated otherwise;
  *   - there is no CPU fallback: without a usable HIP device rlh_init fails and nothing else works.
  *

@@ -440,6 +440,46 @@ def test_percentage_to_gpu_rule(ctx):
         m.free()
 
 
+def test_concurrent_calls_from_threads(ctx):
+    """The reference shares its device handle between rayon workers (transformer.rs:52-53, 783-815).  Calls from several
+    threads on one context and one model, each thread with caches and tensors of its own, give bit for bit what the same calls
+    give one after another."""
+    from concurrent.futures import ThreadPoolExecutor
+    shape = SMALL
+    W = synth_weights(shape, seed=71, std=0.05, norm_ones=False)
+    gm = make_gpu(ctx, shape, W, True)
+    rng = np.random.default_rng(72)
+    jobs = []
+    for i in range(12):
+        n = int(rng.integers(1, 40))
+        jobs.append(([int(t) for t in rng.integers(0, shape.vocab_size, n)], [int(t) for t in rng.integers(0, shape.vocab_size, 4)],
+                     oracle.f32_to_f16_bits(rng.uniform(-1, 1, (7 + i, 64)).astype(f32)), oracle.f32_to_f16_bits(rng.uniform(-1, 1, (33, 64)).astype(f32))))
+
+    def run(job):
+        prompt, follow, a, b = job
+        c = gm.make_caches()
+        out = [gm.forward(prompt, 0, c)]
+        for i, t in enumerate(follow[:2]):
+            out.append(gm.forward([t], len(prompt) + i, c))
+        c2 = c.true_clone()
+        out.append(np.int32(gm.forward_greedy([follow[2]], len(prompt) + 2, c2)))
+        out.append(np.int32(gm.forward_greedy([follow[3]], len(prompt) + 3, c2)))
+        out.append(Tensor.from_numpy(ctx, a).matrix_mul_transposed(Tensor.from_numpy(ctx, b)).to_numpy())
+        out.append(c.read(shape.n_layers - 1, 1, 0))
+        c.free()
+        c2.free()
+        return out
+
+    serial = [run(j) for j in jobs]
+    for _ in range(3):
+        with ThreadPoolExecutor(max_workers=6) as ex:
+            threaded = list(ex.map(run, jobs))
+        for a, b in zip(serial, threaded):
+            for x, y in zip(a, b):
+                assert np.array_equal(x, y)
+    gm.free()
+
+
 def _make_split_gpu(ctx, shape, W, force_f16, p):
     ds = rllama_amd.DataSettings(ctx).percentage_to_gpu(p)
     if force_f16:
