@@ -123,7 +123,8 @@ int  rlh_model_set_prefill_mode(rlh_model *model, int mode);
 /* The layer split rule of src/transformer.rs:262-279: last_layer_on_gpu = round(p * (n_layers - 1)).
  * Layers beyond it have no device storage: rlh_model_set_tensor / get_tensor / rlh_caches_read refuse them. */
 int  rlh_model_layers_on_gpu(const rlh_model *model, int *last_layer_on_gpu);
-/* Bytes of HBM one decode step must read at sequence length T: weights + KV (the roofline's numerator). */
+/* Bytes of HBM one decode step must read at sequence length T: weights + KV (the roofline's numerator); of the resident
+ * layers only, and without the head, for a model split by percentage_to_gpu. */
 int  rlh_model_decode_bytes(const rlh_model *model, int T, uint64_t *bytes);
 
 /* ------------------------------------------------------------------------------------------------

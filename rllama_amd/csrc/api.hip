@@ -549,10 +549,11 @@ extern "C" int rlh_model_layers_on_gpu(const rlh_model *m, int *last_layer_on_gp
 
 extern "C" int rlh_model_decode_bytes(const rlh_model *m, int T, uint64_t *bytes) {
     if (!m || !bytes || T < 1) return fail(RLH_ERR_INVALID, "rlh_model_decode_bytes: bad argument");
-    const uint64_t d = (uint64_t)m->prm.dim, F = (uint64_t)m->prm.ffn_hidden, V = (uint64_t)m->prm.vocab_size, L = (uint64_t)m->prm.n_layers;
+    const uint64_t d = (uint64_t)m->prm.dim, F = (uint64_t)m->prm.ffn_hidden, V = (uint64_t)m->prm.vocab_size, L = (uint64_t)m->n_resident;
     const uint64_t es = m->prm.force_f16 ? 2 : 4;
     const uint64_t head_es = (m->output.p && !m->output.f16) ? 4 : 2;
-    uint64_t b = L * (4 * d * d + 3 * d * F) * es + V * d * head_es;
+    const bool whole = m->n_resident == m->prm.n_layers; // a split model's head is the host's
+    uint64_t b = L * (4 * d * d + 3 * d * F) * es + (whole ? V * d * head_es : 0);
     b += L * 2 * (uint64_t)T * d * es; // K and V rows read
     b += L * 2 * d * es;               // K and V row written
     *bytes = b;
