@@ -544,6 +544,39 @@ def test_hybrid_layer_split(ctx, force_f16, token_by_token):
         gm.free()
 
 
+@pytest.mark.parametrize("force_f16", [True, False], ids=["f16", "f32"])
+def test_each_layer_alone_against_the_oracle(ctx, force_f16):
+    """Config-0 shape, one block at a time: layer l gets the oracle's own stream after layer l - 1 as its input, so every
+    block is compared on identical inputs and no difference is carried from layer to layer (prompt call through the
+    matrix-core path, then single-token calls through the decode kernels, which read the cache planes the prompt call left)."""
+    shape = CONFIG0
+    W = synth_weights(shape, seed=0)
+    om = make_oracle(shape, W, force_f16)
+    gm = make_gpu(ctx, shape, W, force_f16)
+    oc, gc = om.make_caches(), gm.make_caches()
+    prompt = [int(t) for t in rllama_amd.synth_tokens(0, 16, 3, shape.vocab_size)]
+    calls = [(prompt, 0), ([77], 16), ([31000], 17)]
+    # one block on identical inputs: only the order of fp32 additions differs, plus in f16 mode the rounding decisions that flips
+    tol = 2e-3 if force_f16 else 2e-6
+    for toks, start in calls:
+        _, tap = om.forward(toks, start, oc, layer_tap=True)
+        x_in = om.embed(toks)
+        for l in range(shape.n_layers):
+            got = gm.forward_layers(x_in, start, gc, l, l)
+            err = max_rel_err(got, tap[l])
+            assert err < tol, (start, l, err)
+            x_in = tap[l]
+    T = 18
+    for l in (0, shape.n_layers - 1):
+        for which in (0, 1):
+            a, b = gc.read(l, 3, which)[:, :T], oc.read(l, 3, which)[:, :T]
+            # f16 mode: a one-step difference in wk's f16 output passes through the rotation with its pair partner's scale
+            bound = 2 * ulp_f16(b) + 1e-3 * np.abs(b).max() if force_f16 else 1e-5 * np.abs(b).max()
+            assert np.all(np.abs(a - b) <= bound), (l, which, float(np.abs(a - b).max()))
+    gc.free()
+    gm.free()
+
+
 def test_layer_span_on_a_whole_model_equals_its_forward(ctx):
     """On a fully resident model any span runs: two spans back to back give the stream whose norm + head are the logits
     of rlh_forward, and a span over layers that were never set is refused."""
