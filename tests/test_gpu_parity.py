@@ -440,6 +440,42 @@ def test_percentage_to_gpu_rule(ctx):
         m.free()
 
 
+def test_random_small_shapes_against_the_oracle(ctx):
+    """A seeded sweep over model shapes nobody would pick by hand: head dims 16 to 128, one to five heads, ffn widths that are
+    only multiples of 8, odd vocabularies and sequence capacities, prompts up to the capacity, both modes and both prefill
+    paths; logits of the prompt call and of single-token calls after it, and the last head's cache planes, against the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(32):
+        hd = int(rng.choice([16, 32, 64, 128]))
+        H = int(rng.integers(1, 6))
+        ffn = 8 * int(rng.integers(1, 200))
+        vocab = int(rng.integers(5, 700))
+        L = int(rng.integers(1, 4))
+        max_seq = int(rng.integers(4, 150)) if rng.integers(0, 3) else int(rng.integers(150, 700))
+        n_prompt = int(rng.integers(1, max_seq - 2))
+        f16 = bool(rng.integers(0, 2))
+        tbt = bool(rng.integers(0, 2))
+        n_dec = int(min(max_seq - n_prompt - 1, rng.integers(1, 5)))
+        what = f"case {case}: head_dim {hd} heads {H} ffn {ffn} vocab {vocab} layers {L} max_seq {max_seq} prompt {n_prompt} f16 {f16} token-by-token {tbt}"
+        print(what, flush=True)
+        shape = Shape(hd * H, L, H, ffn, vocab, max_seq)
+        W = synth_weights(shape, seed=case, std=0.05, norm_ones=False)
+        om, gm = make_oracle(shape, W, f16), make_gpu(ctx, shape, W, f16)
+        gm.set_prefill_mode(tbt)
+        oc, gc = om.make_caches(), gm.make_caches()
+        tol = TOL_F16 if f16 else TOL_F32
+        toks = [int(t) for t in rng.integers(0, vocab, n_prompt)]
+        assert max_rel_err(gm.forward(toks, 0, gc), om.forward(toks, 0, oc)) < tol, what
+        for i in range(n_dec):
+            t = int(rng.integers(0, vocab))
+            assert max_rel_err(gm.forward([t], n_prompt + i, gc), om.forward([t], n_prompt + i, oc)) < tol, what
+        for l in range(L):
+            for which in (0, 1):
+                assert max_rel_err(gc.read(l, H - 1, which), oc.read(l, H - 1, which)) < tol, what
+        gc.free()
+        gm.free()
+
+
 def test_concurrent_calls_from_threads(ctx):
     """The reference shares its device handle between rayon workers (transformer.rs:52-53, 783-815).  Calls from several
     threads on one context and one model, each thread with caches and tensors of its own, give bit for bit what the same calls
