@@ -854,7 +854,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     A((void **)&S.g, N * F * es);
     if (es == 4) A((void **)&S.u, N * F * es); // f16 mode: w3's epilogue consumes its product on the spot
     A((void **)&S.mm, N * F * es);
-    if (es == 2) A((void **)&S.gemm_ws, PrefillScratch::kGemmWsBytes);
+    A((void **)&S.gemm_ws, PrefillScratch::kGemmWsBytes);
     if (e == hipSuccess) e = hipStreamSynchronize(m->ctx->stream);
     if (e != hipSuccess) {
         S.release();
@@ -1057,6 +1057,8 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
         g.batch = 1;
         g.accumulate = accumulate;
         g.f32_operands = 1;
+        g.workspace = S.gemm_ws;
+        g.workspace_bytes = PrefillScratch::kGemmWsBytes;
         HIP_TRY(launch_gemm_f16(g, kGemmEpiF32, st));
         return RLH_OK;
     };

@@ -393,6 +393,9 @@ static hipError_t launch_dma_f32(const GemmParams &p, int tile, hipStream_t s) {
     case 1: return launch_dma<kGemmEpiF32, 4, 2, 64, 3, true>(p, s);
     case 2: return launch_dma<kGemmEpiF32, 4, 3, 64, 2, true>(p, s);
     case 3: return launch_dma<kGemmEpiF32, 4, 4, 64, 2, true>(p, s);
+    case 5: return launch_dma<kGemmEpiF32, 2, 1, 64, 6, true>(p, s);
+    case 6: return launch_dma<kGemmEpiF32, 1, 1, 64, 10, true, 1>(p, s);
+    case 7: return launch_dma<kGemmEpiF32, 1, 1, 64, 8, true, 2>(p, s);
     default: return hipErrorInvalidValue;
     }
 }
@@ -490,12 +493,13 @@ __global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int
 // in flight, every compute unit busy), their fp32 partial sums go to the caller's workspace and a second small kernel adds
 // them and applies the epilogue.  Returns 1 for "run as one product".
 static int choose_split_k(const GemmParams &p, int tile) {
-    if (p.workspace == nullptr || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.f32_operands) return 1;
-    if (tile != 0 || (p.n % 4) != 0 || (p.ldc % 4) != 0 || p.k % 64 != 0) return 1;
+    if (p.workspace == nullptr || p.batch != 1 || p.k_seg != 0 || p.causal != 0) return 1;
+    const int k_halves = p.k * (p.f32_operands ? 2 : 1);
+    if (tile != 0 || (p.n % 4) != 0 || (p.ldc % 4) != 0 || k_halves % 64 != 0) return 1;
     static const int forced = getenv("RLLAMA_HIP_GEMM_SPLIT_K") ? atoi(getenv("RLLAMA_HIP_GEMM_SPLIT_K")) : 0;
     const int n_cu = device_compute_units();
     const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128);
-    const int k_tiles = p.k / 64;
+    const int k_tiles = k_halves / 64;
     // Worth it while the partial sums (pieces x m x n floats, written and read back) stay small beside the weights: products
     // whose tiles cover at most a quarter of the compute units (measured on the 7B shapes: wq|wk|wv / w1 / w3 on their 86 - 96
     // tiles are faster unsplit on the narrower 128 x 64 tile at any row count, wo / w2 on 32 tiles faster split)
@@ -552,7 +556,7 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         if (blocks <= device_compute_units()) tile = 4;
         // one row tile and few column tiles (a short prompt): half the tile width, so that twice the workgroups stream the
         // weights; the pieces of a split product use it too
-        if (!p.f32_operands && p.m <= 128 && (p.batch == 1 || p.split_k > 1) && (long)((p.n + 127) / 128) * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = p.m <= 32 ? 6 : p.m <= 64 ? 7 : 5;
+        if (p.m <= 128 && (p.batch == 1 || p.split_k > 1) && (long)((p.n + 127) / 128) * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = p.m <= 32 ? 6 : p.m <= 64 ? 7 : 5;
     }
     if (p.f32_operands) {
         if (epilogue != kGemmEpiF32 || ((p.k * 2) % 64) != 0 || (p.k_seg != 0 && ((p.k_seg * 2) % 64) != 0)) return hipErrorInvalidValue;
