@@ -26,7 +26,7 @@ import numpy as np  # noqa: E402
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the dominant kernel (c1: w13 GEMV; c3: w1-shape GEMM; 7B shapes) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs, each scaled by the same counter on a 1 GiB copy kernel (the PMC summary under profiles/ has the commands).
-MEASURED_TRAFFIC = {"c1": 181_001_709, "c3": 186_436_198}
+MEASURED_TRAFFIC = {"c1": 181_001_730, "c3": 186_436_198}
 
 CONFIGS = {
     # name: (dim, n_layers, n_heads, ffn_hidden, vocab, n_prompt, default decode steps)
