@@ -446,6 +446,17 @@ static int choose_tile(const GemmParams &p) {
         const double time = (double)rounds * bms[t] * bns[t] / eff[t];
         if (best < 0 || time < best_t) { best = t; best_t = time; }
     }
+    // fp32 operands run at a sixteenth of the f16 matrix rate, so what counts there is how evenly the tiles fill the compute
+    // units, not the staging: the 128 x 64 tile (tile 5) is a candidate too (7B shape in f32 mode, 384 / 512 prompt rows:
+    // 86 -> 65 / 87 -> 67 ms to the first token; its busy-unit throughput measured 0.93 of the 128 x 128 tile's)
+    // (products with so few tiles that they are cut along K instead keep the 128 x 128 tile that the cut expects)
+    const long tiles128 = (long)((p.n + 127) / 128) * ((p.m + 127) / 128);
+    if (p.f32_operands && p.batch == 1 && p.k_seg == 0 && p.causal == 0 && p.m > 128 && k_halves % 64 == 0 && tiles128 > n_cu / 4) {
+        const long blocks = (long)((p.n + 63) / 64) * ((p.m + 127) / 128);
+        const long rounds = (blocks + n_cu - 1) / n_cu;
+        const double time = (double)rounds * 128 * 64 / 0.93;
+        if (time < best_t) best = 5;
+    }
     return best;
 }
 
