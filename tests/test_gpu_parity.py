@@ -799,6 +799,39 @@ def test_full_size_7b_properties(ctx, n_prompt):
     m.free()
 
 
+@pytest.mark.parametrize("force_f16,prompts", [(True, (5, 40, 130, 300, 1024)), (False, (40, 300, 520))], ids=["f16", "f32"])
+def test_7b_layer_dimensions_against_the_oracle(ctx, force_f16, prompts):
+    """Two layers with the real dimensions of the headline configuration (dim 4096, 32 heads of 128, ffn 11008, vocabulary
+    32000, f16 mode): few enough layers for the oracle, and every kernel runs at the row lengths, tile choices and grids it has
+    in the 7B model.  Prompts of 5, 40, 130, 300 and 1024 tokens take the 32 x 64, 64 x 64, 128 x 64, 128 x 128 and 256 x 192
+    tile paths (the short ones cut along K) and the one-kernel attention at its real head count; single-token calls after each
+    prompt run the decode kernels on the cache the prompt call left.  In f32 mode the same dimensions run the fp32 matrix-core
+    path: 40 rows on the 64 x 64 tile cut along K, 300 on 128 x 128, 520 on the 128 x 64 tile that only fp32 operands choose."""
+    shape = Shape(dim=4096, n_layers=2, n_heads=32, ffn_hidden=11008, vocab_size=32000, max_seq_len=1030)
+    W = synth_weights(shape, seed=0)
+    om = make_oracle(shape, W, force_f16)
+    gm = make_gpu(ctx, shape, W, force_f16)
+    TOL = TOL_F16 if force_f16 else TOL_F32
+    for n_prompt in prompts:
+        toks = [int(t) for t in rllama_amd.synth_tokens(n_prompt, n_prompt, 3, shape.vocab_size)]
+        oc, gc = om.make_caches(), gm.make_caches()
+        print(f"prompt of {n_prompt} tokens", flush=True)
+        want, got = om.forward(toks, 0, oc), gm.forward(toks, 0, gc)
+        assert max_rel_err(got, want) < TOL, (n_prompt, max_rel_err(got, want))
+        top = np.sort(np.where(np.arange(want.size) == 0, 0.0, want))[::-1]                  # the sampler's view: token 0 reads 0.0
+        if top[0] - top[1] > 2 * TOL * np.abs(want).max():                               # a clear winner is the same winner
+            assert int(np.argmax(got[1:])) == int(np.argmax(want[1:]))
+        for i, t in enumerate((17, 31999)):
+            want, got = om.forward([t], n_prompt + i, oc), gm.forward([t], n_prompt + i, gc)
+            assert max_rel_err(got, want) < TOL, (n_prompt, i, max_rel_err(got, want))
+        for l in range(shape.n_layers):
+            for which in (0, 1):
+                a, b = gc.read(l, 31, which), oc.read(l, 31, which)
+                assert max_rel_err(a, b) < TOL, (n_prompt, l, which)
+        gc.free()
+    gm.free()
+
+
 def test_full_size_7b_layer_split(ctx):
     """7B shape split by percentage_to_gpu 0.5 (17 of 32 layers resident): its span calls give bit for bit the stream the same
     span gives on a whole model with the same weights (a prompt call and single-token calls); on the whole model two spans
