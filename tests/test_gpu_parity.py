@@ -832,6 +832,30 @@ def test_7b_layer_dimensions_against_the_oracle(ctx, force_f16, prompts):
     gm.free()
 
 
+@pytest.mark.parametrize("dim,H,F,prompts", [(5120, 40, 13824, (64, 2100)), (8192, 64, 22016, (33, 256))], ids=["13B-dimensions", "65B-dimensions"])
+def test_larger_layer_dimensions_against_the_oracle(ctx, dim, H, F, prompts):
+    """One layer with the dimensions of the 13B and 65B configurations against the oracle: their tile choices and attention
+    grids (40 / 64 heads), and at the 13B dimensions single-token calls at sequence length 2101 and 2102, where the decode
+    attention is split into 17 blocks per head and merged, as in the 2048-token-context configuration."""
+    shape = Shape(dim=dim, n_layers=1, n_heads=H, ffn_hidden=F, vocab_size=4000, max_seq_len=max(prompts) + 4)
+    W = synth_weights(shape, seed=3)
+    om = make_oracle(shape, W, True)
+    gm = make_gpu(ctx, shape, W, True)
+    for n_prompt in prompts:
+        toks = [int(t) for t in rllama_amd.synth_tokens(n_prompt, n_prompt, 3, shape.vocab_size)]
+        oc, gc = om.make_caches(), gm.make_caches()
+        print(f"prompt of {n_prompt} tokens", flush=True)
+        want, got = om.forward(toks, 0, oc), gm.forward(toks, 0, gc)
+        assert max_rel_err(got, want) < TOL_F16, (n_prompt, max_rel_err(got, want))
+        for i, t in enumerate((17, 3999)):
+            want, got = om.forward([t], n_prompt + i, oc), gm.forward([t], n_prompt + i, gc)
+            assert max_rel_err(got, want) < TOL_F16, (n_prompt, i, max_rel_err(got, want))
+        for which in (0, 1):
+            assert max_rel_err(gc.read(0, H - 1, which), oc.read(0, H - 1, which)) < TOL_F16, (n_prompt, which)
+        gc.free()
+    gm.free()
+
+
 def test_full_size_7b_layer_split(ctx):
     """7B shape split by percentage_to_gpu 0.5 (17 of 32 layers resident): its span calls give bit for bit the stream the same
     span gives on a whole model with the same weights (a prompt call and single-token calls); on the whole model two spans
