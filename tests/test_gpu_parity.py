@@ -809,6 +809,9 @@ def test_7b_layer_dimensions_against_the_oracle(ctx, force_f16, prompts):
     path: 40 rows on the 64 x 64 tile cut along K, 300 on 128 x 128, 520 on the 128 x 64 tile that only fp32 operands choose."""
     shape = Shape(dim=4096, n_layers=2, n_heads=32, ffn_hidden=11008, vocab_size=32000, max_seq_len=1030)
     W = synth_weights(shape, seed=0)
+    if not force_f16:  # the embedding table and the head as fp32 tensors, the way the reference holds them (transformer.rs:302-308)
+        for kind in (rllama_amd.TOK_EMB, rllama_amd.OUTPUT):
+            W[(kind, 0)] = W[(kind, 0)].view(np.float16).astype(np.float32)
     om = make_oracle(shape, W, force_f16)
     gm = make_gpu(ctx, shape, W, force_f16)
     TOL = TOL_F16 if force_f16 else TOL_F32
