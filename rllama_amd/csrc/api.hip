@@ -886,14 +886,19 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     }
     const int l_first = span ? span->first : 0, l_last = span ? span->last : P.n_layers - 1;
     const size_t layer_elems = (size_t)H * P.max_seq_len * hd;
+    // norm_w / norm_done: the RMSNorm that follows a residual product, written to S.xn by the product itself where it can
     auto gemm = [&](const void *a, int lda, const void *b, int ldb, void *cc, int ldc, int mm, int nn, int kk, int epi, const float *res,
-                    const void *gate = nullptr) -> int {
+                    const void *gate = nullptr, const float *norm_w = nullptr, int *norm_done = nullptr) -> int {
         GemmParams g{};
         g.a = (const _Float16 *)a;
         g.b = (const _Float16 *)b;
         g.c = cc;
         g.residual = res;
         g.gate = (const _Float16 *)gate;
+        g.norm_w = norm_w;
+        g.norm_out = (_Float16 *)S.xn;
+        g.norm_eps = eps;
+        g.norm_done = norm_done;
         g.m = mm;
         g.n = nn;
         g.k = kk;
@@ -906,11 +911,12 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         HIP_TRY(launch_gemm_f16(g, epi, st));
         return RLH_OK;
     };
+    int normed = 0; // S.xn already holds this layer's attention_norm(S.x): the previous layer's w2 product wrote it
     for (int l = l_first; l <= l_last; l++) {
         Layer &L = m->layers[(size_t)l];
         char *ck = (char *)c->k + (size_t)l * layer_elems * 2;
         char *cv = (char *)c->v + (size_t)l * layer_elems * 2;
-        HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.x, (const float *)L.attn_norm.p, n, d, eps, st));
+        if (!normed) HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.x, (const float *)L.attn_norm.p, n, d, eps, st));
         if ((rc = gemm(S.xn, d, L.wqkv.p, d, S.qkv, 3 * d, n, 3 * d, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
         PrefillRopeParams rp{};
         rp.qkv = S.qkv;
@@ -992,12 +998,16 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
                 HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
             }
         }
-        if ((rc = gemm(S.a, d, L.wo.p, d, S.h, d, n, d, d, kGemmEpiResAddF32, S.x)) != RLH_OK) return rc;     // h = x + wo(att)
-        HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.h, (const float *)L.ffn_norm.p, n, d, eps, st));
+        normed = 0;
+        if ((rc = gemm(S.a, d, L.wo.p, d, S.h, d, n, d, d, kGemmEpiResAddF32, S.x, nullptr, (const float *)L.ffn_norm.p, &normed)) != RLH_OK) return rc; // h = x + wo(att)
+        if (!normed) HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.h, (const float *)L.ffn_norm.p, n, d, eps, st));
         if ((rc = gemm(S.xn, d, L.w1.p, d, S.g, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
         // w3's epilogue applies SiLU(w1 x) * (w3 x) and the f16 rounding points of transformer.rs:557-565 in place of a pass of its own
         if ((rc = gemm(S.xn, d, L.w3.p, d, S.mm, F, n, F, d, kGemmEpiSiluGateF16, nullptr, S.g)) != RLH_OK) return rc;
-        if ((rc = gemm(S.mm, F, L.w2.p, F, S.x, d, n, d, F, kGemmEpiResAddF32, S.h)) != RLH_OK) return rc;    // x = h + w2(...)
+        // x = h + w2(...); the next block's attention_norm rides along where it can
+        normed = 0;
+        const float *next_norm = l < l_last ? (const float *)m->layers[(size_t)l + 1].attn_norm.p : nullptr;
+        if ((rc = gemm(S.mm, F, L.w2.p, F, S.x, d, n, d, F, kGemmEpiResAddF32, S.h, nullptr, next_norm, next_norm ? &normed : nullptr)) != RLH_OK) return rc;
     }
     if (span) {
         HIP_TRY(hipMemcpyAsync(span->x_out, S.x, sizeof(float) * (size_t)n * d, hipMemcpyDeviceToHost, st));

@@ -499,6 +499,51 @@ __global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int
     }
 }
 
+// The same second step for the residual epilogue with the row RMSNorm that follows it: one workgroup per row of C adds the
+// partial sums in the order of the splits, applies the epilogue, keeps the row in registers, and writes the normalised row
+// rounded to f16 as well (the loop structure and the order of additions of rmsnorm_rows_f16_kernel, prefill.hip).
+constexpr int kFinishNormVecs = 8; // rows of up to 256 x 4 x 8 floats
+__global__ __launch_bounds__(256) void gemm_split_finish_norm_kernel(GemmParams p, const float *partial, int splits) {
+    __shared__ float red[16];
+    const size_t per = (size_t)p.m * p.ldc;
+    const int r = blockIdx.x, tid = threadIdx.x, n4 = p.n / 4;
+    const size_t row = (size_t)r * p.ldc;
+    const float4_t *w4 = reinterpret_cast<const float4_t *>(p.norm_w);
+    float4_t xv[kFinishNormVecs];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kFinishNormVecs; j++) {
+        const int i = tid + j * 256;
+        xv[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (i < n4) {
+            const size_t off = row + (size_t)i * 4;
+            float4_t acc = *reinterpret_cast<const float4_t *>(partial + off);
+            for (int z = 1; z < splits; z++) acc += *reinterpret_cast<const float4_t *>(partial + z * per + off);
+            const float4_t res = *reinterpret_cast<const float4_t *>(p.residual + off);
+#pragma unroll
+            for (int e = 0; e < 4; e++) xv[j][e] = res[e] + f16r(acc[e]);
+            *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.c) + off) = xv[j];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) ss = fmaf(xv[j][e], xv[j][e], ss);
+    }
+    ss = block_sum(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)p.n + p.norm_eps);
+    half_t *yr = p.norm_out + (size_t)r * p.n;
+#pragma unroll
+    for (int j = 0; j < kFinishNormVecs; j++) {
+        const int i = tid + j * 256;
+        if (i < n4) {
+            const float4_t wv = w4[i];
+            typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
+            half4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = (half_t)((xv[j][e] * rs) * wv[e]);
+            *reinterpret_cast<half4_t *>(yr + i * 4) = o;
+        }
+    }
+}
+
 // Products with few output tiles (few prompt rows) leave most compute units without a workgroup, and what bounds them is
 // streaming the weights once: the K range is then cut into split_k pieces that run as separate workgroups (more weight bytes
 // in flight, every compute unit busy), their fp32 partial sums go to the caller's workspace and a second small kernel adds
@@ -550,6 +595,12 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         q.workspace = nullptr;
         hipError_t e = launch_gemm_f16_dma(q, kGemmEpiF32, s);
         if (e != hipSuccess) return e;
+        if (epilogue == kGemmEpiResAddF32 && p_in.norm_w != nullptr && p_in.norm_out != nullptr && p_in.norm_done != nullptr &&
+            p_in.n <= 256 * 4 * kFinishNormVecs && !(getenv("RLLAMA_HIP_FINISH_NORM") && atoi(getenv("RLLAMA_HIP_FINISH_NORM")) == 0)) {
+            hipLaunchKernelGGL(gemm_split_finish_norm_kernel, dim3(p_in.m), dim3(256), 0, s, p_in, (const float *)p_in.workspace, splits);
+            *p_in.norm_done = 1;
+            return hipGetLastError();
+        }
         switch (epilogue) {
         case kGemmEpiF16: return launch_split_finish<kGemmEpiF16>(p_in, splits, s);
         case kGemmEpiF32: return launch_split_finish<kGemmEpiF32>(p_in, splits, s);

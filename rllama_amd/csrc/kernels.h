@@ -101,6 +101,14 @@ struct GemmParams {
     size_t workspace_bytes;
     int f32_operands;       // 1: a and b point to fp32 data (f32 mode); m, n, k, lda, ldb, strides and k_seg count elements
                             //    all the same.  Needs k % 32 == 0 and the kGemmEpiF32 epilogue.
+    // Optional (kGemmEpiResAddF32, fast path): the RMSNorm that follows the residual add (transformer.rs:443 after :442, :432 of
+    // the next block after :445).  Where the launcher adds up split-K partial sums anyway, that kernel also writes
+    // norm_out = f16(rmsnorm(C row) * norm_w) and sets *norm_done = 1 at launch; otherwise it leaves both alone and the
+    // caller runs the norm kernel itself.  Same arithmetic, same order of additions either way.
+    const float *norm_w;    // [n]
+    _Float16 *norm_out;     // [m x n], row stride n
+    float norm_eps;
+    int *norm_done;         // host flag
 };
 
 hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s);

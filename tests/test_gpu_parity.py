@@ -3,6 +3,8 @@
 Tolerances are the ones the task states: logits within max relative error 1e-2 for f16 weights and 1e-4 for f32
 (relative to the largest |logit|), greedy token ids identical on config 0.  Op-level checks are tighter.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -254,8 +256,17 @@ def test_prefill_short_prompt_split_k(ctx):
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
     for n in (100, 5):
         oc, gc = om.make_caches(), gm.make_caches()
-        assert max_rel_err(gm.forward(toks[:n], 0, gc), om.forward(toks[:n], 0, oc)) < TOL_F16
+        got = gm.forward(toks[:n], 0, gc)
+        assert max_rel_err(got, om.forward(toks[:n], 0, oc)) < TOL_F16
         assert max_rel_err(gm.forward(toks[n:n + 1], n, gc), om.forward(toks[n:n + 1], n, oc)) < TOL_F16
+        # the kernel that adds the partial sums of wo / w2 also writes the RMSNorm that follows; with that switched off the
+        # norm runs as a kernel of its own: same arithmetic in the same order, so the same bits
+        os.environ["RLLAMA_HIP_FINISH_NORM"] = "0"
+        try:
+            g2 = gm.make_caches()
+            assert np.array_equal(gm.forward(toks[:n], 0, g2), got)
+        finally:
+            del os.environ["RLLAMA_HIP_FINISH_NORM"]
     gm.free()
 
 
