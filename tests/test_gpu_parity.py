@@ -115,6 +115,31 @@ def test_matrix_mul_transposed_multi_row(ctx):
         Tensor.from_numpy(ctx, np.zeros((2, 8), f32)).matrix_mul_transposed(Tensor.from_numpy(ctx, np.zeros((2, 8), np.uint16)))
 
 
+def test_random_products_against_float64(ctx):
+    """A seeded sweep over product shapes: 1 to 1300 rows (the values around the tile edges more often), ragged column counts,
+    K any multiple of 8 (f16) or 4 (fp32) up to 4800; f16 results within one f16 step of the float64 product plus fp32
+    summation noise, fp32 results within summation noise."""
+    rng = np.random.default_rng(77)
+    for case in range(48):
+        f16 = bool(rng.integers(0, 2))
+        m = int(rng.choice([1, 2, 3, 7, 31, 32, 33, 64, 65, 127, 128, 129, 255, 257, 500, 1024, 1100])) if rng.integers(0, 2) else int(rng.integers(1, 1300))
+        n = int(rng.integers(1, 3000)) if rng.integers(0, 4) else int(rng.choice([64, 128, 192, 256, 3072, 4096]))
+        k = (8 if f16 else 4) * int(rng.integers(1, 600)) if rng.integers(0, 2) else 64 * int(rng.integers(1, 70))
+        what = f"case {case}: f16 {f16}, {m} x {n} x {k}"
+        print(what, flush=True)
+        a = rng.uniform(-1, 1, (m, k)).astype(f32)
+        b = rng.uniform(-1, 1, (n, k)).astype(f32)
+        if f16:
+            a, b = a.astype(np.float16), b.astype(np.float16)
+            got = Tensor.from_numpy(ctx, a.view(np.uint16)).matrix_mul_transposed(Tensor.from_numpy(ctx, b.view(np.uint16))).to_numpy().view(np.float16)
+        else:
+            got = Tensor.from_numpy(ctx, a).matrix_mul_transposed(Tensor.from_numpy(ctx, b)).to_numpy()
+        want = a.astype(np.float64) @ b.astype(np.float64).T
+        mag = np.abs(a.astype(np.float64)) @ np.abs(b.astype(np.float64)).T
+        tol = np.abs(want) * 2.0 ** -10 + mag * 1.6e-6 + 1e-6 if f16 else mag * 3e-6 + 1e-7
+        assert got.shape == want.shape and np.all(np.abs(got.astype(np.float64) - want) <= tol), what
+
+
 def test_elementwise_ops(ctx):
     rng = np.random.default_rng(6)
     for rows, cols in [(1, 1), (3, 5), (64, 64), (37, 300)]:
