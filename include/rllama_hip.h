@@ -243,7 +243,11 @@ int  rlh_rope_inplace(rlh_tensor *x, int n_heads, int head_dim, int pos);
 /* One kernel of the token step, cycling through the layers so that every launch streams different weights.
  * which: 0 = attention_norm + wq|wk|wv + RoPE + cache write, 1 = single-query attention at sequence length T,
  * 2 = wo + residual, 3 = ffn_norm + w1|w3 + SiLU*gate, 4 = w2 + residual, 5 = final norm + output head.
- * bytes_per_launch (may be NULL): the algorithmic bytes of one launch (weights once + vectors). */
+ * bytes_per_launch (may be NULL): the algorithmic bytes of one launch (weights once + vectors).
+ * The launches use the model's token-step state and activation buffers as they are and leave them overwritten (position
+ * T - 1, a fixed token id), and which = 0 writes the K / V rows of position T - 1 of every layer of `caches`: use caches
+ * made for the measurement.  A greedy loop in progress is ended (rlh_decode_greedy refuses until the next
+ * rlh_forward_greedy / rlh_generate_greedy). */
 int  rlh_model_time_kernel(rlh_model *model, rlh_caches *caches, int which, int T, int iters, float *us_per_launch,
                            uint64_t *bytes_per_launch);
 /* Isolated GEMV y = W x, W [rows x k] of w_dtype, x f32, cycling through n_buffers distinct weight buffers

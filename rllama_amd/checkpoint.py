@@ -299,6 +299,12 @@ class Checkpoint:
         """rows x cols f16 bits of one shard's piece, read row by row like src/tensor.rs:2452-2480."""
         if b.stride < 1:
             raise ValueError(f"invalid stride {b.stride}")
+        # The pickle is untrusted input (BININT / BININT2 are signed): check every extent before it sizes a read, and
+        # take the storage key only as a file name inside consolidated.NN/data/ (src/data_source.rs:105-111).
+        if b.rows <= 0 or b.cols <= 0 or b.offset < 0 or b.nitems < 0 or b.offset + b.rows * b.cols > b.nitems:
+            raise ValueError(f"{b.tensor_name}: shape {b.rows}x{b.cols} at offset {b.offset} does not fit its storage of {b.nitems} items")
+        if not b.src_path or "/" in b.src_path or "\\" in b.src_path or b.src_path in (".", ".."):
+            raise ValueError(f"{b.tensor_name}: storage key {b.src_path!r} is not a plain file name")
         fn = os.path.join(self.path, f"consolidated.{shard:02d}", "data", b.src_path)
         want = b.rows * b.cols
         arr = np.fromfile(fn, dtype="<u2", count=want, offset=2 * b.offset)
@@ -369,18 +375,20 @@ def _binint(v: int) -> bytes:
 
 
 def pickle_state_dict(entries: Sequence[Tuple[str, str, Tuple[int, ...]]]) -> bytes:
-    """entries: (tensor name, storage key, shape).  One dict, one MARK ... SETITEMS batch."""
+    """entries: (tensor name, storage key, shape[, storage offset, storage items]).  One dict, one MARK ... SETITEMS batch.
+    The two optional fields default to 0 and the shape's element count (tests use them to write damaged files)."""
     out = bytearray(b"\x80\x02\x7d\x28")
-    for name, key, shape in entries:
+    for name, key, shape, *rest in entries:
         if len(shape) not in (1, 2):
             raise ValueError("only 1-D and 2-D tensors")
-        nitems = int(np.prod(shape))
+        offset = int(rest[0]) if len(rest) > 0 else 0
+        nitems = int(rest[1]) if len(rest) > 1 else int(np.prod(shape))
         out += _binunicode(name)
         out += b"ctorch._utils\n_rebuild_tensor_v2\n"
         out += b"\x28"                                             # MARK: args tuple
         out += b"\x28" + _binunicode("storage") + b"ctorch\nHalfStorage\n" + _binunicode(key) + _binunicode("cpu") + _binint(nitems) + b"\x74"
         out += b"\x51"                                             # BINPERSID
-        out += _binint(0)                                          # storage offset
+        out += _binint(offset)                                     # storage offset
         if len(shape) == 2:
             out += _binint(shape[0]) + _binint(shape[1]) + b"\x86" + _binint(shape[1]) + _binint(1) + b"\x86"
         else:

@@ -1442,6 +1442,9 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
         default: *bytes_per_launch = V * d * (m->output.f16 ? 2 : 4) + d * 4 + d * 4 + V * 4; break;
         }
     }
+    // the timed launches run on the model's own token-step state and buffers: whatever greedy loop was in progress is over
+    m->next_pos = -1;
+    m->greedy_caches = nullptr;
     HIP_TRY(launch_set_state(m->state, T - 1, 3 % m->prm.vocab_size, 1, st));
     hipEvent_t e0 = nullptr, e1 = nullptr;
     HIP_TRY(hipEventCreate(&e0));

@@ -15,6 +15,7 @@
 #include "rllama_hip.hpp"
 
 #include <cerrno>
+#include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <fstream>
@@ -409,6 +410,18 @@ inline HalfMatrix load_from_pieces(const DataSource &src, const std::string &nam
     HalfMatrix m;
     for (const auto &b : builders) {
         if (b.stride < 1) throw std::runtime_error(name + ": invalid stride");
+        // The pickle is untrusted input: BININT / BININT2 are signed, so every extent is checked before it sizes a buffer
+        // or addresses a file (the reference reaches the same values through usize casts and slice bounds, which panic).
+        if (b.rows <= 0 || b.cols <= 0 || b.offset < 0 || b.nitems < 0 || b.rows > INT32_MAX || b.cols > INT32_MAX ||
+            b.offset + b.rows * b.cols > b.nitems) {
+            throw std::runtime_error(name + ": shape " + std::to_string(b.rows) + "x" + std::to_string(b.cols) + " at offset " + std::to_string(b.offset) +
+                                     " does not fit its storage of " + std::to_string(b.nitems) + " items");
+        }
+        // the storage key names a file inside consolidated.NN/data/ (src/data_source.rs:105-111), never a path
+        if (b.src_path.empty() || b.src_path.find('/') != std::string::npos || b.src_path.find('\\') != std::string::npos || b.src_path == "." ||
+            b.src_path == "..") {
+            throw std::runtime_error(name + ": storage key '" + b.src_path + "' is not a plain file name");
+        }
         if (direction == FromPiecesDirection::Rows) {
             if (b.cols != builders[0].cols) throw std::runtime_error(name + ": pieces differ in cols");
             m.rows += b.rows;

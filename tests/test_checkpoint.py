@@ -256,3 +256,51 @@ def test_synthetic_checkpoint_matches_the_generator(tmp_path):
     emb = c.load_f16_bits("tok_embeddings.weight", ck.FROM_PIECES_COLS)
     assert np.array_equal(emb, rllama_amd.synth_normal_f16(3, rllama_amd.TOK_EMB, 0, 96 * 64).reshape(96, 64))
     assert np.all(c.load_f16_bits("layers.0.ffn_norm.weight", ck.FROM_PIECES_ROWS, True) == 0x3C00)
+
+
+def _hostile_dir(tmp_path, tag, entries_by_shard, files):
+    """A model directory whose data.pkl files hold `entries_by_shard[i]` and whose data/ folders hold `files[i]`."""
+    path = tmp_path / tag
+    path.mkdir()
+    (path / "params.json").write_text(json.dumps({"dim": 8, "n_heads": 2, "n_layers": 1, "norm_eps": 1e-6, "vocab_size": 4}))
+    for i, entries in enumerate(entries_by_shard):
+        sd = path / f"consolidated.{i:02d}"
+        (sd / "data").mkdir(parents=True)
+        (sd / "data.pkl").write_bytes(ck.pickle_state_dict(entries))
+        for key, n in files[i].items():
+            (sd / "data" / key).write_bytes(np.arange(n, dtype="<u2").tobytes())
+    return str(path)
+
+
+@pytest.mark.parametrize("tag,entries,msg", [
+    # negative extents (BININT is signed, src/unpickler.rs:414): one shard claims 6 columns, the other -4, so the sum (2) would
+    # size the joined matrix while the first shard still copies 6 columns per row
+    ("mixed_sign_cols", [[("w", "0", (3, 6))], [("w", "0", (3, -4))]], "invalid stride|does not fit its storage"),
+    ("negative_rows", [[("w", "0", (-2, 4))]], "does not fit its storage"),
+    ("zero_cols", [[("w", "0", (0,))]], "does not fit its storage"),
+    ("negative_cols_1d", [[("w", "0", (-4,), 0, 8)]], "does not fit its storage"),
+    ("negative_offset", [[("w", "0", (2, 4), -1, 8)]], "does not fit its storage"),
+    ("past_the_storage", [[("w", "0", (2, 4), 4, 8)]], "does not fit its storage"),
+    # the storage key must stay a file name inside consolidated.NN/data/
+    ("dotdot_key", [[("w", "../../params.json", (1, 2))]], "not a plain file name"),
+    ("absolute_key", [[("w", "/etc/hostname", (1, 2))]], "not a plain file name"),
+])
+def test_damaged_checkpoints_fail_cleanly_in_both_readers(tmp_path, tag, entries, msg):
+    """Extents and storage keys come from the pickle unchecked; both readers must refuse them before sizing a buffer or
+    opening a path (the reference panics on the same inputs: usize casts of negative i64 and slice bounds)."""
+    import subprocess
+    from rllama_amd import build
+    files = [{"0": 64} for _ in entries]
+    path = _hostile_dir(tmp_path, tag, entries, files)
+    with pytest.raises(ValueError, match=msg):
+        ck.Checkpoint(path).load_f16_bits("w", ck.FROM_PIECES_COLS)
+    r = subprocess.run([build.build_host(), "--inspect", path], capture_output=True, text=True, timeout=60)
+    import re
+    assert r.returncode == 1 and re.search(msg, r.stderr), (r.returncode, r.stderr)
+
+
+def test_offset_and_item_count_are_honoured(tmp_path):
+    """A piece that starts inside its storage file reads from there (storage offset in elements, src/tensor.rs:2452-2480)."""
+    path = _hostile_dir(tmp_path, "off", [[("w", "0", (2, 3), 5, 16)]], [{"0": 16}])
+    got = ck.Checkpoint(path).load_f16_bits("w", ck.FROM_PIECES_ROWS)
+    assert np.array_equal(got, np.arange(5, 11, dtype=np.uint16).reshape(2, 3))
