@@ -147,6 +147,8 @@ def main() -> int:
     ap.add_argument("--kernels-only", action="store_true",
                     help="skip the token loop and the CPU baseline: only the per-kernel timing loops (short runs for "
                          "rocprofv3 --pmc passes)")
+    ap.add_argument("--kernel", default=None, help="with --kernels-only: time only this token-step kernel (a name from the output's \"kernels\")")
+    ap.add_argument("--kernel-T", type=int, default=None, help="with --kernels-only: the sequence length the attention kernel sees")
     ap.add_argument("--percentage-to-gpu", type=float, default=1.0,
                     help="below 1: time the device's share of a layer-split model (rlh_forward_layers over layers "
                          "0..=round(p * (n_layers - 1)), stream handed over from and to host memory on every call)")
@@ -176,7 +178,7 @@ def main() -> int:
     dim, n_layers, n_heads, ffn, vocab, n_prompt, dflt_steps = CONFIGS[args.config]
     K = args.steps if args.steps is not None else dflt_steps
     W = max(0, args.warmup)
-    max_seq = n_prompt + max(K, W) + 1
+    max_seq = max(n_prompt + max(K, W) + 1, (args.kernel_T or 0) + 1)
 
     ctx = ra.Context(0, verbose=False)
     info = ctx.device_info()
@@ -241,9 +243,11 @@ def main() -> int:
 
     if args.kernels_only:
         caches = model.make_caches()
-        T_mid = n_prompt + K // 2
+        T_mid = args.kernel_T if args.kernel_T else n_prompt + K // 2
         out = {"kernels_only": True, "T": T_mid, "kernels": {}}
         for which, name in enumerate(ra.Transformer.STEP_KERNELS):
+            if args.kernel and name != args.kernel:
+                continue
             us, nbytes = model.time_kernel(which, T_mid, args.kernel_iters, caches)
             out["kernels"][name] = {"us": round(us, 2), "bytes": nbytes}
         print(json.dumps(out))

@@ -236,6 +236,40 @@ int  rlh_rmsnorm(rlh_tensor *y, const rlh_tensor *x, const rlh_tensor *w, double
 /* apply_rotary_emb (src/transformer.rs:823-856) on one [n_heads x head_dim] f32 row at position pos, in place. */
 int  rlh_rope_inplace(rlh_tensor *x, int n_heads, int head_dim, int pos);
 
+/* The steps of the attention block and of the token loop that the reference runs on the host (its OpenCL backend has no
+ * call for them); here they are device kernels of the forward, exported one by one so that each can be checked alone.
+ * "Cache planes" are one layer's K and V cache as the forward holds them: two tensors [n_heads * max_seq_len x head_dim]
+ * of one dtype (f16 or f32), row h * max_seq_len + t = head h, position t -- the transpose of the reference's per-head
+ * [head_dim x max_seq_len] (src/transformer.rs:143-154).  head_dim is 16, 32, 64 or 128. */
+/* Tensor::add (src/tensor.rs:573-593) as the residual adds use it (src/transformer.rs:442, 445): dst = a + b, f32. */
+int  rlh_add(rlh_tensor *dst, const rlh_tensor *a, const rlh_tensor *b);
+/* FeedForward's gate (src/transformer.rs:557-565): dst = silu(gate) * up, formed in f32 (src/tensor.rs:822-832, 722-734);
+ * f16 tensors are read as f16 and the product is rounded to f16 once. */
+int  rlh_silu_mul(rlh_tensor *dst, const rlh_tensor *gate, const rlh_tensor *up);
+/* One token's cache update (src/transformer.rs:704-761 with seq_len 1): RoPE on q (in place) and on k at position pos,
+ * then k and v into the cache planes at pos (rounded to f16 for f16 planes).  q, k, v: f32, n_heads * head_dim elements. */
+int  rlh_rope_kvwrite(rlh_tensor *q, const rlh_tensor *k, const rlh_tensor *v, rlh_tensor *cache_k, rlh_tensor *cache_v, int n_heads,
+                      int max_seq_len, int pos);
+/* Single-query attention over positions 0..T-1 of the cache planes (src/transformer.rs:762-781 with seq_len 1: scores
+ * src/tensor.rs:1923-1983, softmax :479-494, P.V :1282-1475): out = softmax(q K^T / sqrt(head_dim)) V per head.
+ * q (after RoPE) and out: f32, n_heads * head_dim elements; round_out = the f16 rounding point before wo (:793-796).
+ * n_splits: blocks per head the positions are shared between, 1..64; 0 = the forward's own choice for T.
+ * The softmax subtracts the running maximum: equal to the reference's exp(s) / sum exp(s) wherever that is finite, and
+ * finite where the reference overflows to NaN (scores above ln(FLT_MAX)). */
+int  rlh_attn_decode(rlh_tensor *out, const rlh_tensor *q, const rlh_tensor *cache_k, const rlh_tensor *cache_v, int n_heads, int max_seq_len,
+                     int T, int n_splits, int round_out);
+/* The attention block of a multi-token forward at start_pos 0 between the projections and wo (src/transformer.rs:704-796):
+ * RoPE on the q and k columns of qkv, k and v into the cache planes at positions 0..n-1, causal attention per head, heads
+ * concatenated and rounded to f16.  qkv: f16 [n x 3 dim] (columns [0, dim) wq's output, [dim, 2 dim) wk's, [2 dim, 3 dim)
+ * wv's); out: f16 [n x dim]; f16 cache planes; head_dim 64 or 128 (the one-kernel matrix-core form). */
+int  rlh_attn_prefill(rlh_tensor *out, const rlh_tensor *qkv, rlh_tensor *cache_k, rlh_tensor *cache_v, int n_heads, int max_seq_len);
+/* TokenSampler::sample with top_k = 1 (src/token_sampler.rs:83-174) on device logits (an f32 vector), as the greedy
+ * entry points run it: logits * (1 / temperature) when temperature > 0 (:99-102), token 0's value becomes 0 (:112-123),
+ * un-shifted softmax, first of the descending probabilities with NaN last (:124-147).  While the softmax sum is finite that
+ * is the largest scaled logit (lowest id among equal ones); once it is not (a scaled logit above ln(FLT_MAX), a NaN, or
+ * the sum itself overflowing) every probability is 0 or NaN and the pick is token 0. */
+int  rlh_argmax_greedy(const rlh_tensor *logits, float temperature, int32_t *token);
+
 /* ------------------------------------------------------------------------------------------------
  * Measurement aids (no reference counterpart; src/benches/benchmark.rs times the CPU/OpenCL ops with criterion).
  * Both time `iters` back-to-back launches with HIP events on the launch stream.

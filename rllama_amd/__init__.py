@@ -369,6 +369,42 @@ class Tensor:
     def rope_inplace(self, n_heads: int, head_dim: int, pos: int) -> None:
         check(self._lib.rlh_rope_inplace(self._h, n_heads, head_dim, pos))
 
+    # the host-side steps of the reference's attention block and token loop, as device ops
+    def add(self, other: "Tensor") -> "Tensor":
+        """Tensor::add (src/tensor.rs:573-593), f32."""
+        out = self._like()
+        check(self._lib.rlh_add(out._h, self._h, other._h))
+        return out
+
+    def silu_mul(self, up: "Tensor") -> "Tensor":
+        """silu(self) * up with one rounding for f16 tensors (src/transformer.rs:557-565)."""
+        out = self._like()
+        check(self._lib.rlh_silu_mul(out._h, self._h, up._h))
+        return out
+
+    def rope_kvwrite(self, k: "Tensor", v: "Tensor", cache_k: "Tensor", cache_v: "Tensor", n_heads: int, max_seq_len: int, pos: int) -> None:
+        """self = q: RoPE on q (in place) and k at pos; k and v into the cache planes at pos (src/transformer.rs:704-761)."""
+        check(self._lib.rlh_rope_kvwrite(self._h, k._h, v._h, cache_k._h, cache_v._h, n_heads, max_seq_len, pos))
+
+    def attn_decode(self, cache_k: "Tensor", cache_v: "Tensor", n_heads: int, max_seq_len: int, T: int, n_splits: int = 0,
+                    round_out: bool = False) -> "Tensor":
+        """self = q after RoPE: single-query attention over positions 0..T-1 of the cache planes (src/transformer.rs:762-781)."""
+        out = Tensor.zeros(self.ctx, 1, self._rows * self._cols, TensorDType.Float32)
+        check(self._lib.rlh_attn_decode(out._h, self._h, cache_k._h, cache_v._h, n_heads, max_seq_len, T, n_splits, 1 if round_out else 0))
+        return out
+
+    def attn_prefill(self, cache_k: "Tensor", cache_v: "Tensor", n_heads: int, max_seq_len: int) -> "Tensor":
+        """self = qkv f16 [n x 3 dim]: RoPE, cache write and causal attention of a prompt (src/transformer.rs:704-796) -> f16 [n x dim]."""
+        out = Tensor.zeros(self.ctx, self._rows, self._cols // 3, TensorDType.Float16)
+        check(self._lib.rlh_attn_prefill(out._h, self._h, cache_k._h, cache_v._h, n_heads, max_seq_len))
+        return out
+
+    def argmax_greedy(self, temperature: float = 1.0) -> int:
+        """TokenSampler::sample at top_k = 1 on device logits (src/token_sampler.rs:83-174)."""
+        tok = C.c_int32()
+        check(self._lib.rlh_argmax_greedy(self._h, float(temperature), C.byref(tok)))
+        return int(tok.value)
+
     def free(self) -> None:
         if getattr(self, "_h", None):
             if self.ctx._h:

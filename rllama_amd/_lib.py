@@ -86,6 +86,12 @@ SIGNATURES = {
     "rlh_gemv": (C.c_int, [_vp, _vp, _vp, C.c_int, C.c_int]),
     "rlh_rmsnorm": (C.c_int, [_vp, _vp, _vp, C.c_double, C.c_int]),
     "rlh_rope_inplace": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int]),
+    "rlh_add": (C.c_int, [_vp, _vp, _vp]),
+    "rlh_silu_mul": (C.c_int, [_vp, _vp, _vp]),
+    "rlh_rope_kvwrite": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int]),
+    "rlh_attn_decode": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "rlh_attn_prefill": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, C.c_int]),
+    "rlh_argmax_greedy": (C.c_int, [_vp, C.c_float, _i32p]),
     "rlh_model_time_kernel": (C.c_int, [_vp, _vp, C.c_int, C.c_int, C.c_int, _fp, C.POINTER(C.c_uint64)]),
     "rlh_time_gemv": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _fp]),
     "rlh_synth_normal_f16": (None, [C.c_uint64, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_double, C.POINTER(C.c_uint16)]),

@@ -5,7 +5,7 @@
 // -> rlh_ctx; Transformer (transformer.rs:17-34) -> rlh_model; TransformerCaches (transformer.rs:111-113)
 // -> rlh_caches; OpenCLTensor (tensor_opencl_support.rs:23-38) -> rlh_tensor.
 #include "../../include/rllama_hip.h"
-#include "kernels.h"
+#include "api_internal.h"
 #include "synth.h"
 
 #include <hip/hip_runtime.h>
@@ -29,7 +29,8 @@ using namespace rlh;
 // ------------------------------------------------------------------------------------------------
 static thread_local std::string g_last_error;
 
-static int fail(int code, const char *fmt, ...) {
+namespace rlh {
+int fail(int code, const char *fmt, ...) {
     char buf[512];
     va_list ap;
     va_start(ap, fmt);
@@ -38,19 +39,8 @@ static int fail(int code, const char *fmt, ...) {
     g_last_error = buf;
     return code;
 }
-
-namespace rlh {
-int set_error(int code, const char *msg) { return fail(code, "%s", msg); } // for the library's other translation units
+int set_error(int code, const char *msg) { return fail(code, "%s", msg); }
 } // namespace rlh
-
-#define HIP_TRY(expr)                                                                                     \
-    do {                                                                                                  \
-        hipError_t _e = (expr);                                                                           \
-        if (_e != hipSuccess) {                                                                           \
-            return fail(_e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "%s failed: %s (%s:%d)",   \
-                        #expr, hipGetErrorString(_e), __FILE__, __LINE__);                                \
-        }                                                                                                 \
-    } while (0)
 
 extern "C" const char *rlh_last_error(void) { return g_last_error.c_str(); }
 extern "C" int rlh_abi_version(void) { return RLH_ABI_VERSION; }
@@ -58,14 +48,6 @@ extern "C" int rlh_abi_version(void) { return RLH_ABI_VERSION; }
 // ------------------------------------------------------------------------------------------------
 // objects
 // ------------------------------------------------------------------------------------------------
-struct rlh_ctx {
-    int device = 0;
-    int verbose = 0;
-    hipStream_t stream = nullptr;
-    hipDeviceProp_t prop;
-    std::recursive_mutex mu;
-};
-
 struct Weight {
     void *p = nullptr;
     int rows = 0, cols = 0;
@@ -119,9 +101,13 @@ struct rlh_model {
     int32_t *prompt_dev = nullptr;
     int prompt_cap = 0;
     float *attn_ws = nullptr;
-    int max_splits = 32;
-    int attn_single_max = 384; // sequence lengths up to this use one block per head (measured: one block 5.6 us at 384 positions against 6.5 us split + merge; 7.1 against 6.4 at 512)
+    unsigned *attn_tickets = nullptr; // [n_heads] arrival counters of the in-kernel merge (zero between launches)
+    int max_splits = kAttnDecodeMaxSplits;
+    int attn_single_max = 384; // sequence lengths up to this use one block per head
     int attn_chunk = 128;      // positions per block beyond that
+    int attn_merge_mode = 2;   // how the blocks of a split sequence are merged (AttnDecodeParams::merge_mode)
+    bool capturing = false;    // a decode step is being recorded into a HIP graph
+    bool attn_lds_stage = getenv("RLLAMA_HIP_ATTN_LDS") && atoi(getenv("RLLAMA_HIP_ATTN_LDS")) != 0; // comparison variant of the decode attention
     int stream_weights = 1;
     PrefillScratch pf;
     int prefill_mode = 0; // 0: matrix-core prefill where available (f16 mode), 1: token by token
@@ -151,24 +137,6 @@ struct rlh_caches {
     int f16 = 0;
     // one captured decode step (token step + greedy pick) per attention grid shape, replayed by the greedy loops
     std::map<int, hipGraphExec_t> step_graphs;
-};
-
-struct rlh_tensor {
-    rlh_ctx *ctx = nullptr;
-    void *p = nullptr;
-    int rows = 0, cols = 0, dtype = RLH_F16;
-    size_t esize() const { return dtype == RLH_F16 ? 2 : 4; }
-    size_t count() const { return (size_t)rows * cols; }
-};
-
-struct rlh_event {
-    rlh_ctx *ctx = nullptr;
-    hipEvent_t ev = nullptr;
-};
-
-struct CtxLock {
-    std::lock_guard<std::recursive_mutex> g;
-    explicit CtxLock(rlh_ctx *c) : g(c->mu) { (void)hipSetDevice(c->device); }
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -217,6 +185,7 @@ extern "C" void rlh_shutdown(rlh_ctx *ctx) {
         (void)hipStreamSynchronize(ctx->stream);
         (void)hipStreamDestroy(ctx->stream);
     }
+    ops_release(ctx);
     delete ctx;
 }
 
@@ -295,6 +264,10 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
         const int v = atoi(e);
         if (v >= 0) m->attn_single_max = v;
     }
+    if (const char *e = getenv("RLLAMA_HIP_ATTN_MERGE")) {
+        const int v = atoi(e);
+        if (v >= 0 && v <= 2) m->attn_merge_mode = v;
+    }
     // transformer.rs:266-268
     m->last_layer_on_gpu = (int)std::round(m->prm.percentage_to_gpu * (float)(prm->n_layers - 1));
     m->n_resident = m->last_layer_on_gpu + 1;
@@ -355,7 +328,8 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     B((void **)&m->state, sizeof(DecodeState));
     B((void **)&m->out_tokens, sizeof(int32_t) * m->out_cap);
     B((void **)&m->prompt_dev, sizeof(int32_t) * m->prompt_cap);
-    B((void **)&m->attn_ws, sizeof(float) * (size_t)prm->n_heads * m->max_splits * (hd + 2));
+    B((void **)&m->attn_ws, sizeof(float) * attn_decode_workspace_floats(prm->n_heads, hd, m->max_splits));
+    B((void **)&m->attn_tickets, sizeof(unsigned) * (size_t)prm->n_heads);
     if (rc == RLH_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(RLH_ERR_HIP, "rlh_model_create: hipDeviceSynchronize failed");
     if (rc != RLH_OK) {
         rlh_model_free(m);
@@ -382,7 +356,7 @@ extern "C" void rlh_model_free(rlh_model *m) {
     free_weight(m->norm);
     free_weight(m->output);
     m->pf.release();
-    void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws};
+    void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws, m->attn_tickets};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -672,15 +646,7 @@ extern "C" int rlh_caches_read(const rlh_caches *c, int layer, int head, int whi
 // ------------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------------
-static int attn_splits(const rlh_model *m, int T) {
-    // One block per (head, split).  A block streams its share of the cache alone, so short sequences stay in one
-    // block per head (no merge launch); longer ones are cut into chunks of about attn_chunk positions.
-    if (T <= m->attn_single_max) return 1;
-    int S = (T + m->attn_chunk - 1) / m->attn_chunk;
-    if (S < 1) S = 1;
-    if (S > m->max_splits) S = m->max_splits;
-    return S;
-}
+static int attn_splits(const rlh_model *m, int T) { return attn_splits_rule(T, m->attn_single_max, m->attn_chunk, m->max_splits); }
 
 enum StepKernel { kStepQkv = 0, kStepAttn = 1, kStepWo = 2, kStepW13 = 3, kStepW2 = 4, kStepHead = 5 };
 
@@ -760,6 +726,7 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         a.cache_v = cv;
         a.cache_f16 = c->f16;
         a.state = m->state;
+        a.pos_host = m->capturing ? -1 : T_host - 1; // a captured step is replayed at later positions: it reads the device state
         a.n_heads = P.n_heads;
         a.head_dim = m->head_dim;
         a.max_seq_len = P.max_seq_len;
@@ -767,6 +734,11 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         a.out = m->att;
         a.round_out = f16;
         a.workspace = m->attn_ws;
+        a.tickets = m->attn_tickets;
+        a.merge_mode = m->attn_merge_mode;
+        a.chunk_hint = (((T_host + a.n_splits - 1) / a.n_splits) + 15) & ~15;
+        a.lds_stage = m->attn_lds_stage && !m->capturing && c->f16 && (m->head_dim == 128 || m->head_dim == 64) && a.merge_mode == 2 &&
+                      (size_t)a.chunk_hint * m->head_dim * 4 <= 128 * 1024;
         HIP_TRY(launch_attn_decode(a, st));
         break;
     }
@@ -1212,7 +1184,8 @@ extern "C" int rlh_forward(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     return RLH_OK;
 }
 
-extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, int32_t *next_token) {
+// forward + the device pick at top_k = 1 on logits * scale
+static int forward_greedy_scaled(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, int32_t *next_token, float scale) {
     int rc = check_forward_args(m, c, tokens, n, start_pos, "rlh_forward_greedy");
     if (rc != RLH_OK) return rc;
     if (!next_token) return fail(RLH_ERR_INVALID, "rlh_forward_greedy: next_token is NULL");
@@ -1220,12 +1193,16 @@ extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *to
     hipStream_t st = m->ctx->stream;
     rc = enqueue_forward(m, c, tokens, n, start_pos);
     if (rc != RLH_OK) return rc;
-    HIP_TRY(launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st));
+    HIP_TRY(launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st, scale));
     HIP_TRY(hipMemcpyAsync(next_token, m->out_tokens, sizeof(int32_t), hipMemcpyDeviceToHost, st));
     HIP_TRY(hipStreamSynchronize(st));
     m->next_pos = start_pos + n;
     m->greedy_caches = c;
     return RLH_OK;
+}
+
+extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, int32_t *next_token) {
+    return forward_greedy_scaled(m, c, tokens, n, start_pos, next_token, 1.0f);
 }
 
 extern "C" int rlh_forward_layers(rlh_model *m, rlh_caches *c, const float *x_in, int n, int start_pos, int first_layer, int last_layer,
@@ -1284,10 +1261,12 @@ extern "C" int rlh_forward_sample(rlh_model *m, rlh_caches *c, const int32_t *to
                                   const int32_t *existing_tokens, int n_existing, float u, int32_t *token, float *prob) {
     if (!sp || !token) return fail(RLH_ERR_INVALID, "rlh_forward_sample: NULL argument");
     if (sp->top_k == 1) {
-        // one candidate: the draw cannot choose.  Which one it is does not depend on temperature (> 0 keeps the order, and
-        // token 0 sits at exactly 0 either way) nor on the penalty (it only reaches token 0, whose value is then shifted to 0),
-        // so the device argmax with the token-0 rule decides (token_sampler.rs:99-147).
-        const int rc = rlh_forward_greedy(m, c, tokens, n, start_pos, token);
+        // one candidate: the draw cannot choose.  Which one it is does not depend on the penalty (it only reaches token 0,
+        // whose value is then shifted to 0); the temperature matters only through what it does to the un-shifted softmax
+        // (scaled logits beyond ln(FLT_MAX) turn probabilities into NaN), so the device pick runs on the scaled logits
+        // (token_sampler.rs:99-147).
+        const float scale = sp->temperature > 0.0f ? 1.0f / sp->temperature : 1.0f;
+        const int rc = forward_greedy_scaled(m, c, tokens, n, start_pos, token, scale);
         if (rc == RLH_OK && prob) *prob = 1.0f; // v.1 / total_p with a single candidate (:170)
         return rc;
     }
@@ -1316,7 +1295,9 @@ static int enqueue_decode_step(rlh_model *m, rlh_caches *c, int T_host) {
     if (it == c->step_graphs.end()) {
         hipGraph_t graph = nullptr;
         HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        m->capturing = true;
         int rc = enqueue_token_step(m, c, T_host, true);
+        m->capturing = false;
         hipError_t e = rc == RLH_OK ? launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st) : hipSuccess;
         hipError_t e2 = hipStreamEndCapture(st, &graph);
         if (rc != RLH_OK || e != hipSuccess || e2 != hipSuccess) {
@@ -1517,255 +1498,6 @@ extern "C" int rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int rou
     HIP_TRY(e);
     HIP_TRY(e2);
     *us_per_launch = ms * 1000.0f / (float)iters;
-    return RLH_OK;
-}
-
-// ------------------------------------------------------------------------------------------------
-// op level
-// ------------------------------------------------------------------------------------------------
-extern "C" int rlh_tensor_alloc(rlh_ctx *ctx, int rows, int cols, int dtype, rlh_tensor **out) {
-    if (!ctx || !out || rows <= 0 || cols <= 0 || (dtype != RLH_F16 && dtype != RLH_F32)) return fail(RLH_ERR_INVALID, "rlh_tensor_alloc: bad argument");
-    *out = nullptr;
-    CtxLock lock(ctx);
-    rlh_tensor *t = new rlh_tensor();
-    t->ctx = ctx;
-    t->rows = rows;
-    t->cols = cols;
-    t->dtype = dtype;
-    hipError_t e = hipMalloc(&t->p, t->count() * t->esize());
-    if (e == hipSuccess) e = hipMemsetAsync(t->p, 0, t->count() * t->esize(), ctx->stream);
-    if (e != hipSuccess) {
-        if (t->p) (void)hipFree(t->p);
-        delete t;
-        return fail(e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "rlh_tensor_alloc: %s", hipGetErrorString(e));
-    }
-    *out = t;
-    return RLH_OK;
-}
-
-extern "C" int rlh_tensor_upload(rlh_ctx *ctx, const void *host, int rows, int cols, int cols_capacity, int dtype, rlh_tensor **out) {
-    if (!host || cols_capacity < cols) return fail(RLH_ERR_INVALID, "rlh_tensor_upload: bad argument");
-    int rc = rlh_tensor_alloc(ctx, rows, cols, dtype, out);
-    if (rc != RLH_OK) return rc;
-    CtxLock lock(ctx);
-    rlh_tensor *t = *out;
-    const size_t es = t->esize();
-    hipError_t e = hipMemcpy2DAsync(t->p, (size_t)cols * es, host, (size_t)cols_capacity * es, (size_t)cols * es, (size_t)rows,
-                                    hipMemcpyHostToDevice, ctx->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream); // the host buffer is the caller's again on return
-    if (e != hipSuccess) {
-        rlh_tensor_free(t);
-        *out = nullptr;
-        return fail(RLH_ERR_HIP, "rlh_tensor_upload: %s", hipGetErrorString(e));
-    }
-    return RLH_OK;
-}
-
-extern "C" int rlh_tensor_download(rlh_tensor *t, void *host, int cols_capacity, rlh_event **ev) {
-    if (!t || !host || cols_capacity < t->cols) return fail(RLH_ERR_INVALID, "rlh_tensor_download: bad argument");
-    CtxLock lock(t->ctx);
-    const size_t es = t->esize();
-    HIP_TRY(hipMemcpy2DAsync(host, (size_t)cols_capacity * es, t->p, (size_t)t->cols * es, (size_t)t->cols * es, (size_t)t->rows,
-                             hipMemcpyDeviceToHost, t->ctx->stream));
-    if (ev) {
-        int rc = rlh_event_record(t->ctx, ev);
-        if (rc != RLH_OK) return rc;
-    } else {
-        HIP_TRY(hipStreamSynchronize(t->ctx->stream));
-    }
-    return RLH_OK;
-}
-
-extern "C" void rlh_tensor_free(rlh_tensor *t) {
-    if (!t) return;
-    CtxLock lock(t->ctx);
-    (void)hipStreamSynchronize(t->ctx->stream);
-    if (t->p) (void)hipFree(t->p);
-    delete t;
-}
-
-extern "C" int rlh_tensor_shape(const rlh_tensor *t, int *rows, int *cols, int *dtype) {
-    if (!t) return fail(RLH_ERR_INVALID, "rlh_tensor_shape: NULL tensor");
-    if (rows) *rows = t->rows;
-    if (cols) *cols = t->cols;
-    if (dtype) *dtype = t->dtype;
-    return RLH_OK;
-}
-
-extern "C" int rlh_event_record(rlh_ctx *ctx, rlh_event **out) {
-    if (!ctx || !out) return fail(RLH_ERR_INVALID, "rlh_event_record: NULL argument");
-    CtxLock lock(ctx);
-    rlh_event *ev = new rlh_event();
-    ev->ctx = ctx;
-    hipError_t e = hipEventCreate(&ev->ev);
-    if (e == hipSuccess) e = hipEventRecord(ev->ev, ctx->stream);
-    if (e != hipSuccess) {
-        if (ev->ev) (void)hipEventDestroy(ev->ev);
-        delete ev;
-        return fail(RLH_ERR_HIP, "rlh_event_record: %s", hipGetErrorString(e));
-    }
-    *out = ev;
-    return RLH_OK;
-}
-
-extern "C" int rlh_event_wait(rlh_event *ev) {
-    if (!ev) return fail(RLH_ERR_INVALID, "rlh_event_wait: NULL event");
-    hipError_t e = hipEventSynchronize(ev->ev);
-    (void)hipEventDestroy(ev->ev);
-    delete ev;
-    if (e != hipSuccess) return fail(RLH_ERR_HIP, "rlh_event_wait: %s", hipGetErrorString(e));
-    return RLH_OK;
-}
-
-extern "C" int rlh_event_elapsed_ms(rlh_event *start, rlh_event *stop, float *ms) {
-    if (!start || !stop || !ms) return fail(RLH_ERR_INVALID, "rlh_event_elapsed_ms: NULL argument");
-    HIP_TRY(hipEventSynchronize(stop->ev));
-    HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
-    return RLH_OK;
-}
-
-extern "C" void rlh_event_free(rlh_event *ev) {
-    if (!ev) return;
-    if (ev->ev) (void)hipEventDestroy(ev->ev);
-    delete ev;
-}
-
-static int same_shape(const rlh_tensor *a, const rlh_tensor *b) { return a->rows == b->rows && a->cols == b->cols && a->dtype == b->dtype; }
-
-extern "C" int rlh_copy_inplace(rlh_tensor *dst, const rlh_tensor *src) {
-    if (!dst || !src || !same_shape(dst, src)) return fail(RLH_ERR_INVALID, "rlh_copy_inplace: shape/dtype mismatch");
-    CtxLock lock(dst->ctx);
-    // a plain copy kernel (the reference's copy_inplace is a kernel too); also the calibration point for HBM counters
-    HIP_TRY(launch_convert(dst->p, dst->dtype == RLH_F16, src->p, src->dtype == RLH_F16, dst->count(), dst->ctx->stream));
-    return RLH_OK;
-}
-
-extern "C" int rlh_transpose_from(rlh_tensor *dst, const rlh_tensor *src) {
-    if (!dst || !src || dst->rows != src->cols || dst->cols != src->rows || dst->dtype != src->dtype) {
-        return fail(RLH_ERR_INVALID, "rlh_transpose_from: shape/dtype mismatch");
-    }
-    CtxLock lock(dst->ctx);
-    HIP_TRY(launch_transpose(dst->p, src->p, src->rows, src->cols, src->dtype == RLH_F16, dst->ctx->stream));
-    return RLH_OK;
-}
-
-extern "C" int rlh_hadamard_product_inplace(rlh_tensor *dst, const rlh_tensor *src) {
-    if (!dst || !src || !same_shape(dst, src)) return fail(RLH_ERR_INVALID, "rlh_hadamard_product_inplace: shape/dtype mismatch");
-    CtxLock lock(dst->ctx);
-    HIP_TRY(launch_hadamard(dst->p, src->p, dst->count(), dst->dtype == RLH_F16, dst->ctx->stream));
-    return RLH_OK;
-}
-
-extern "C" int rlh_silu_inplace(rlh_tensor *t) {
-    if (!t) return fail(RLH_ERR_INVALID, "rlh_silu_inplace: NULL tensor");
-    CtxLock lock(t->ctx);
-    HIP_TRY(launch_silu(t->p, t->count(), t->dtype == RLH_F16, t->ctx->stream));
-    return RLH_OK;
-}
-
-extern "C" int rlh_gemv(rlh_tensor *y, const rlh_tensor *w, const rlh_tensor *x, int round_x, int round_y) {
-    if (!y || !w || !x) return fail(RLH_ERR_INVALID, "rlh_gemv: NULL argument");
-    if (x->dtype != RLH_F32 || y->dtype != RLH_F32) return fail(RLH_ERR_INVALID, "rlh_gemv: x and y must be f32");
-    if (x->rows != 1 || y->rows != 1 || x->cols != w->cols || y->cols != w->rows) return fail(RLH_ERR_INVALID, "rlh_gemv: shape mismatch");
-    const int vec = w->dtype == RLH_F16 ? 8 : 4;
-    if (w->cols % vec != 0) return fail(RLH_ERR_UNSUPPORTED, "rlh_gemv: k must be a multiple of %d", vec);
-    CtxLock lock(y->ctx);
-    GemvParams p{};
-    p.w = w->p;
-    p.w_is_f16 = w->dtype == RLH_F16;
-    p.x = (const float *)x->p;
-    p.x_f16 = round_x ? 1 : 0;
-    p.round_y = round_y ? 1 : 0;
-    p.y = (float *)y->p;
-    p.n_rows = w->rows;
-    p.k = w->cols;
-    p.stream_weights = 1;
-    HIP_TRY(launch_gemv(p, kEpiStore, y->ctx->stream));
-    return RLH_OK;
-}
-
-extern "C" int rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tensor *src, const rlh_tensor *other) {
-    if (!dst || !src || !other) return fail(RLH_ERR_INVALID, "rlh_matrix_mul_inplace_transposed: NULL argument");
-    if (src->cols != other->cols) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication %dx%d vs %dx%d", src->rows, src->cols, other->rows, other->cols);
-    if (src->dtype != other->dtype || dst->dtype != src->dtype) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication, different dtypes");
-    if (dst->rows != src->rows) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication, different number of rows");
-    if (dst->cols != other->rows) return fail(RLH_ERR_INVALID, "Invalid matrix multiplication, different number of cols");
-    const int f16 = src->dtype == RLH_F16;
-    if (src->cols % (f16 ? 8 : 4) != 0) return fail(RLH_ERR_UNSUPPORTED, "rlh_matrix_mul_inplace_transposed: k must be a multiple of %d", f16 ? 8 : 4);
-    CtxLock lock(dst->ctx);
-    hipStream_t st = dst->ctx->stream;
-    const int n = src->rows, k = src->cols, mrows = other->rows;
-    if (n > 1 && (f16 || k % 32 == 0)) {
-        // more than one row: the matrix-core GEMM (fp32 operands need whole K-tiles of 32, else the per-row path below)
-        GemmParams g{};
-        g.a = (const _Float16 *)src->p;
-        g.b = (const _Float16 *)other->p;
-        g.c = dst->p;
-        g.m = n;
-        g.n = mrows;
-        g.k = k;
-        g.lda = k;
-        g.ldb = k;
-        g.ldc = mrows;
-        g.batch = 1;
-        g.f32_operands = f16 ? 0 : 1;
-        HIP_TRY(launch_gemm_f16(g, f16 ? kGemmEpiF16 : kGemmEpiF32, st));
-        return RLH_OK;
-    }
-    float *xf = nullptr, *yf = nullptr;
-    HIP_TRY(hipMalloc((void **)&xf, sizeof(float) * (size_t)n * k));
-    hipError_t e = hipMalloc((void **)&yf, sizeof(float) * (size_t)n * mrows);
-    if (e == hipSuccess) e = launch_convert(xf, 0, src->p, f16, (uint64_t)n * k, st);
-    for (int r = 0; e == hipSuccess && r < n; r++) {
-        GemvParams p{};
-        p.w = other->p;
-        p.w_is_f16 = f16;
-        p.x = xf + (size_t)r * k;
-        p.x_f16 = f16;
-        p.round_y = f16;
-        p.y = yf + (size_t)r * mrows;
-        p.n_rows = mrows;
-        p.k = k;
-        p.stream_weights = 0;
-        e = launch_gemv(p, kEpiStore, st);
-    }
-    if (e == hipSuccess) e = launch_convert(dst->p, f16, yf, 0, (uint64_t)n * mrows, st);
-    hipError_t e2 = hipStreamSynchronize(st);
-    if (xf) (void)hipFree(xf);
-    if (yf) (void)hipFree(yf);
-    HIP_TRY(e);
-    HIP_TRY(e2);
-    return RLH_OK;
-}
-
-extern "C" int rlh_rmsnorm(rlh_tensor *y, const rlh_tensor *x, const rlh_tensor *w, double eps, int round_y) {
-    if (!y || !x || !w) return fail(RLH_ERR_INVALID, "rlh_rmsnorm: NULL argument");
-    if (x->dtype != RLH_F32 || y->dtype != RLH_F32 || w->dtype != RLH_F32) return fail(RLH_ERR_INVALID, "rlh_rmsnorm: f32 tensors only");
-    if (!same_shape(x, y) || w->rows != 1 || w->cols != x->cols) return fail(RLH_ERR_INVALID, "rlh_rmsnorm: shape mismatch");
-    CtxLock lock(y->ctx);
-    HIP_TRY(launch_rmsnorm_rows((float *)y->p, (const float *)x->p, (const float *)w->p, x->rows, x->cols, (float)eps, round_y, y->ctx->stream));
-    return RLH_OK;
-}
-
-extern "C" int rlh_rope_inplace(rlh_tensor *x, int n_heads, int head_dim, int pos) {
-    if (!x || x->dtype != RLH_F32 || n_heads <= 0 || head_dim <= 0 || (head_dim % 2) != 0 || pos < 0 || x->count() != (size_t)n_heads * head_dim) {
-        return fail(RLH_ERR_INVALID, "rlh_rope_inplace: bad argument");
-    }
-    CtxLock lock(x->ctx);
-    std::vector<float2> tab((size_t)head_dim / 2);
-    for (int j = 0; j < head_dim / 2; j++) {
-        const double freq = 1.0 / std::pow(10000.0, (double)j * 2.0 / (double)head_dim);
-        const double ang = freq * (double)pos;
-        tab[(size_t)j] = make_float2((float)std::cos(ang), (float)std::sin(ang));
-    }
-    float2 *dev = nullptr;
-    HIP_TRY(hipMalloc((void **)&dev, tab.size() * sizeof(float2)));
-    hipError_t e = hipMemcpyAsync(dev, tab.data(), tab.size() * sizeof(float2), hipMemcpyHostToDevice, x->ctx->stream);
-    if (e == hipSuccess) e = launch_rope_row((float *)x->p, n_heads, head_dim, dev, x->ctx->stream);
-    hipError_t e2 = hipStreamSynchronize(x->ctx->stream);
-    (void)hipFree(dev);
-    HIP_TRY(e);
-    HIP_TRY(e2);
     return RLH_OK;
 }
 

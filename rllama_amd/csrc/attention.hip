@@ -10,22 +10,15 @@
 // consumed (independent loads in flight hide the memory latency; a single query leaves nothing to reuse).  Every lane group keeps a running
 // (max, sum, weighted V) triple (the max-subtracted form equals the reference's exp(s) / sum exp(s)
 // wherever that is finite), so the main loop has no block-wide synchronisation; the groups' triples are
-// merged once at the end through LDS.  Long sequences are split over several blocks per head
-// (grid.y); their partial triples go to a workspace and a small second kernel merges them.
+// merged once at the end through LDS.  A sequence is split over several blocks per head (grid.y); every block
+// publishes its partial triple to a workspace and takes a ticket, and the block that draws the last ticket of its
+// head merges the partial triples (in split order, so the result does not depend on which block that was).
 #include "kernels.h"
 #include "device_utils.h"
 
 namespace rlh {
 
-#ifndef RLH_ATTN_THREADS
-#define RLH_ATTN_THREADS 512
-#endif
-#ifndef RLH_ATTN_BATCH
-#define RLH_ATTN_BATCH 4
-#endif
-constexpr int kAttnThreads = RLH_ATTN_THREADS;
-constexpr int kAttnWaves = kAttnThreads / kWave;
-constexpr int kAttnBatch = RLH_ATTN_BATCH; // cache rows of K and of V loaded together per lane
+constexpr int kAttnMaxSplits = 64;
 
 template <typename CT>
 __device__ __forceinline__ void load8(const CT *p, float (&out)[8]) {
@@ -62,8 +55,33 @@ __device__ __forceinline__ void unpack8(const uint4_t *raw, float (&out)[8]) {
     }
 }
 
-template <typename CT, int kHeadDim>
-__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeParams p) {
+// How the partial triples of a split sequence travel from the blocks that make them to the block that merges them.
+enum AttnMergeMode {
+    kMergeSeparate = 0, // a second kernel merges (attn_merge_kernel)
+    kMergeFenced = 1,   // last block of a head merges; release / acquire fences at device scope around the ticket
+    kMergeThrough = 2   // last block of a head merges; the partials are stored and loaded at device scope (write-through /
+                        // cache-bypassing accesses), the stores only waited for before the ticket
+};
+
+template <int kMode>
+__device__ __forceinline__ void publish(float *dst, float v) {
+    if constexpr (kMode == kMergeThrough) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *dst = v;
+}
+template <int kMode>
+__device__ __forceinline__ float collect(const float *src) {
+    if constexpr (kMode == kMergeThrough) return __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else return *src;
+}
+
+// kThreads threads per block, kBatch cache rows of K and of V loaded together per lane before any is consumed.
+// kLds: the block's K and V rows are first moved into LDS as whole tiles (direct global -> LDS loads) and consumed from
+// there; otherwise they go from memory straight into registers.
+template <typename CT, int kHeadDim, int kThreads, int kBatch, int kMode, bool kLds = false>
+__global__ __launch_bounds__(kThreads) void attn_decode_kernel(AttnDecodeParams p) {
+    constexpr int kAttnThreads = kThreads;
+    constexpr int kAttnWaves = kThreads / kWave;
+    constexpr int kAttnBatch = kBatch;
     constexpr int kRawPerRow = sizeof(CT) == 2 ? 1 : 2;
     constexpr int kLanesPerPos = kHeadDim / 8;        // each lane owns 8 consecutive dims
     constexpr int kPosPerWave = kWave / kLanesPerPos; // positions per wave step
@@ -79,7 +97,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
     const int head = blockIdx.x;
     const int split = blockIdx.y;
     const int S = gridDim.y;
-    const int T = p.state->pos + 1;
+    const int T = (p.pos_host >= 0 ? p.pos_host : p.state->pos) + 1;
     int chunk = (T + S - 1) / S;
     chunk = (chunk + 15) & ~15;
     const int t0 = split * chunk;
@@ -100,6 +118,30 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.0f;
 
+    // LDS-staged form (f16 caches): the block's rows [t0, t1) of K and of V are contiguous in memory; every wavefront moves
+    // 1 KiB pieces of them (each lane names its own 16 bytes, clamped to the last valid row) and the block waits once.
+    extern __shared__ uint4_t lds_kv[];
+    const int rows_cap = chunk;                                      // the launcher sized the LDS for this many rows
+    const uint4_t *lds_k = lds_kv;
+    const uint4_t *lds_v = lds_kv + (size_t)rows_cap * kLanesPerPos; // 16-byte words per row = kLanesPerPos
+    if constexpr (kLds) {
+        static_assert(!kLds || sizeof(CT) == 2, "LDS staging is built for f16 caches");
+        const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_kv;
+        const int rows = t1 > t0 ? t1 - t0 : 0;
+        const int words = rows * kLanesPerPos;           // 16-byte words of one tile
+        const int pieces = (words + kWave - 1) / kWave;  // 1 KiB pieces
+        const half_t *ksrc = reinterpret_cast<const half_t *>(p.cache_k) + ((size_t)head * p.max_seq_len + t0) * kHeadDim;
+        const half_t *vsrc = reinterpret_cast<const half_t *>(p.cache_v) + ((size_t)head * p.max_seq_len + t0) * kHeadDim;
+        const int wv = __builtin_amdgcn_readfirstlane(wave);
+        for (int pc = wv; pc < pieces; pc += kAttnWaves) {
+            const int w = min(pc * kWave + lane, words - 1);
+            dma16(ksrc + (size_t)w * 8, lds_base + (unsigned)pc * 1024u);
+            dma16(vsrc + (size_t)w * 8, lds_base + (unsigned)(rows_cap * kLanesPerPos * 16) + (unsigned)pc * 1024u);
+        }
+        wait_vmcnt<0>();
+        __syncthreads();
+    }
+
     // this lane group's positions: t0 + (wave + g * kAttnWaves) * kPosPerWave + sub, g = 0, 1, ...
     // kAttnBatch steps are loaded together (2 * kAttnBatch independent 16-byte loads in flight per lane)
     const int stride = kAttnWaves * kPosPerWave;
@@ -113,8 +155,14 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
             const size_t off = (size_t)min(t + u * stride, t_safe) * kHeadDim;
 #pragma unroll
             for (int w = 0; w < kRawPerRow; w++) {
-                kraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(kbase + off) + 16 * w);
-                vraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(vbase + off) + 16 * w);
+                if constexpr (kLds) {
+                    const int r = min(t + u * stride, t_safe) - t0;
+                    kraw[u][w] = lds_k[r * kLanesPerPos + dl];
+                    vraw[u][w] = lds_v[r * kLanesPerPos + dl];
+                } else {
+                    kraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(kbase + off) + 16 * w);
+                    vraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(vbase + off) + 16 * w);
+                }
             }
         }
         // the scores of the batch first (independent of each other), then one new maximum and one rescale for the batch:
@@ -181,18 +229,78 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodePar
         } else {
             float *ws = p.workspace + ((size_t)head * S + split) * (kHeadDim + 2);
             if (tid == 0) {
-                ws[0] = M;
-                ws[1] = L;
+                publish<kMode>(ws + 0, M);
+                publish<kMode>(ws + 1, L);
             }
-            ws[2 + tid] = O;
+            publish<kMode>(ws + 2 + tid, O);
+        }
+    }
+    if constexpr (kMode != kMergeSeparate) {
+        if (S == 1) return;
+        // ---- the block that draws the last ticket of this head merges the head's partial triples ----
+        __shared__ int is_last;
+        // every writer makes its stores visible to the device before the block's ticket is drawn
+        if constexpr (kMode == kMergeFenced) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        else { // the write-through stores have left the wavefront (and been acknowledged) before the ticket is drawn
+            asm volatile("" ::: "memory");
+            wait_vmcnt<0>();
+            asm volatile("" ::: "memory");
+        }
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned prev = __hip_atomic_fetch_add(p.tickets + head, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = prev == (unsigned)(S - 1);
+            if (last) __hip_atomic_store(p.tickets + head, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
+            is_last = last;
+        }
+        __syncthreads();
+        if (!is_last) return;
+        if constexpr (kMode == kMergeFenced) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        // Every wavefront forms the splits' weights for itself (lane s holds split s), and the first partial outputs are
+        // requested before those weights are needed: one memory latency for the whole merge, no exchange through LDS.
+        const float *wh = p.workspace + (size_t)head * S * (kHeadDim + 2);
+        float ms = -INFINITY, ls = 0.0f;
+        if (lane < S) {
+            ms = collect<kMode>(wh + (size_t)lane * (kHeadDim + 2));
+            ls = collect<kMode>(wh + (size_t)lane * (kHeadDim + 2) + 1);
+        }
+        constexpr int kMergeBatch = 8;
+        const int col = tid < kHeadDim ? tid : 0; // threads beyond head_dim compute along and store nothing
+        float ob[kMergeBatch];
+#pragma unroll
+        for (int u = 0; u < kMergeBatch; u++) ob[u] = u < S ? collect<kMode>(wh + (size_t)u * (kHeadDim + 2) + 2 + col) : 0.0f;
+        const float Mh = wave_max(ms);
+        const float fh = ls > 0.0f ? expf(ms - Mh) : 0.0f;
+        const float Lh = wave_sum(ls * fh);
+        float O = 0.0f;
+        for (int s0 = 0; s0 < S; s0 += kMergeBatch) {
+            float cur[kMergeBatch];
+#pragma unroll
+            for (int u = 0; u < kMergeBatch; u++) cur[u] = ob[u];
+            if (s0 + kMergeBatch < S) {
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; u++) {
+                    const int s2 = s0 + kMergeBatch + u;
+                    ob[u] = s2 < S ? collect<kMode>(wh + (size_t)s2 * (kHeadDim + 2) + 2 + col) : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kMergeBatch; u++) {
+                const int s2 = s0 + u; // in split order: the sum does not depend on which block merges
+                if (s2 < S) O = fmaf(cur[u], __shfl(fh, s2, kWave), O);
+            }
+        }
+        if (tid < kHeadDim) {
+            const float o = O / Lh;
+            p.out[head * kHeadDim + tid] = p.round_out ? f16r(o) : o;
         }
     }
 }
 
-// Merges the per-split triples of one head: grid = heads, block = max(head_dim, 64) threads.  The first wavefront
-// turns the (max, sum) pairs into one weight per split (one load per lane, wave reductions); then thread j sums
-// the weighted partial outputs of dim j with independent loads.
-constexpr int kAttnMaxSplits = 64;
+// Merges the per-split triples of one head as a kernel of its own (kMergeSeparate): grid = heads, block = max(head_dim, 64)
+// threads.  The first wavefront turns the (max, sum) pairs into one weight per split (one load per lane, wave
+// reductions); then thread j sums the weighted partial outputs of dim j with independent loads.  The in-kernel merge above
+// does the same arithmetic in the same order.
 __global__ void attn_merge_kernel(const float *workspace, int n_splits, int head_dim, float *out, int round_out) {
     __shared__ float wgt[kAttnMaxSplits];
     __shared__ float l_total;
@@ -231,27 +339,72 @@ __global__ void attn_merge_kernel(const float *workspace, int n_splits, int head
     }
 }
 
-template <typename CT>
+template <typename CT, int kThreads, int kBatch, int kMode>
 static hipError_t launch_attn_t(const AttnDecodeParams &p, hipStream_t s) {
     dim3 grid(p.n_heads, p.n_splits);
     switch (p.head_dim) {
-    case 128: hipLaunchKernelGGL((attn_decode_kernel<CT, 128>), grid, dim3(kAttnThreads), 0, s, p); break;
-    case 64: hipLaunchKernelGGL((attn_decode_kernel<CT, 64>), grid, dim3(kAttnThreads), 0, s, p); break;
-    case 32: hipLaunchKernelGGL((attn_decode_kernel<CT, 32>), grid, dim3(kAttnThreads), 0, s, p); break;
-    case 16: hipLaunchKernelGGL((attn_decode_kernel<CT, 16>), grid, dim3(kAttnThreads), 0, s, p); break;
+    case 128: hipLaunchKernelGGL((attn_decode_kernel<CT, 128, kThreads, kBatch, kMode>), grid, dim3(kThreads), 0, s, p); break;
+    case 64: hipLaunchKernelGGL((attn_decode_kernel<CT, 64, kThreads, kBatch, kMode>), grid, dim3(kThreads), 0, s, p); break;
+    case 32: hipLaunchKernelGGL((attn_decode_kernel<CT, 32, kThreads, kBatch, kMode>), grid, dim3(kThreads), 0, s, p); break;
+    case 16: hipLaunchKernelGGL((attn_decode_kernel<CT, 16, kThreads, kBatch, kMode>), grid, dim3(kThreads), 0, s, p); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
+// LDS-staged variant (kept for comparison): f16 cache, head_dim 64 / 128, write-through merge
+static hipError_t launch_attn_lds(const AttnDecodeParams &p, hipStream_t s) {
+    const int chunk = p.chunk_hint;
+    const size_t lds = (size_t)2 * chunk * p.head_dim * 2;
+    dim3 grid(p.n_heads, p.n_splits);
+    auto go = [&](auto kern) -> hipError_t {
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, p);
+        return hipGetLastError();
+    };
+    if (p.head_dim == 128) return go(attn_decode_kernel<half_t, 128, 512, 4, kMergeThrough, true>);
+    return go(attn_decode_kernel<half_t, 64, 512, 4, kMergeThrough, true>);
+}
+
+template <typename CT, int kMode>
+static hipError_t launch_attn_m(const AttnDecodeParams &p, hipStream_t s) {
+    // Block shape by the positions a block covers (an upper bound from the host's view of the sequence length): 512 threads
+    // cover 64 * 512 / head_dim positions per step of the loop, and the rows of kBatch steps are in flight together, so up to
+    // 8 steps run as one batch (one exposed memory latency); longer chunks loop with batches of 4.
+    const int chunk = p.chunk_hint > 0 ? p.chunk_hint : p.max_seq_len;
+    const int per_step = 8 * 512 / p.head_dim;
+    if (chunk <= 2 * per_step) return launch_attn_t<CT, 512, 2, kMode>(p, s);
+    if (chunk > 4 * per_step && chunk <= 8 * per_step) return launch_attn_t<CT, 512, 8, kMode>(p, s);
+    return launch_attn_t<CT, 512, 4, kMode>(p, s);
+}
+
 hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s) {
     if (p.n_splits < 1 || p.n_splits > kAttnMaxSplits) return hipErrorInvalidValue;
     if (p.n_splits > 1 && p.workspace == nullptr) return hipErrorInvalidValue;
-    hipError_t e = p.cache_f16 ? launch_attn_t<half_t>(p, s) : launch_attn_t<float>(p, s);
-    if (e != hipSuccess || p.n_splits == 1) return e;
+    if (p.n_splits > 1 && p.merge_mode != kMergeSeparate && p.tickets == nullptr) return hipErrorInvalidValue;
+    if (p.lds_stage) {
+        // needs the exact chunk the kernel will compute (host position known), an f16 cache and room in LDS
+        if (p.pos_host < 0 || !p.cache_f16 || (p.head_dim != 128 && p.head_dim != 64) || p.merge_mode != kMergeThrough ||
+            (size_t)2 * p.chunk_hint * p.head_dim * 2 > 128 * 1024)
+            return hipErrorInvalidValue;
+        return launch_attn_lds(p, s);
+    }
+    hipError_t e;
+    switch (p.merge_mode) {
+    case kMergeSeparate: e = p.cache_f16 ? launch_attn_m<half_t, kMergeSeparate>(p, s) : launch_attn_m<float, kMergeSeparate>(p, s); break;
+    case kMergeFenced: e = p.cache_f16 ? launch_attn_m<half_t, kMergeFenced>(p, s) : launch_attn_m<float, kMergeFenced>(p, s); break;
+    case kMergeThrough: e = p.cache_f16 ? launch_attn_m<half_t, kMergeThrough>(p, s) : launch_attn_m<float, kMergeThrough>(p, s); break;
+    default: return hipErrorInvalidValue;
+    }
+    if (e != hipSuccess || p.n_splits == 1 || p.merge_mode != kMergeSeparate) return e;
     hipLaunchKernelGGL(attn_merge_kernel, dim3(p.n_heads), dim3(p.head_dim < kWave ? kWave : p.head_dim), 0, s, p.workspace, p.n_splits, p.head_dim, p.out,
                        p.round_out);
     return hipGetLastError();
 }
+
+size_t attn_decode_workspace_floats(int n_heads, int head_dim, int n_splits) { return (size_t)n_heads * n_splits * (head_dim + 2); }
 
 } // namespace rlh

@@ -59,17 +59,26 @@ struct AttnDecodeParams {
     const void *cache_k;      // this layer: [n_heads x max_seq_len x head_dim]
     const void *cache_v;
     int cache_f16;
-    const DecodeState *state; // T = state->pos + 1
+    const DecodeState *state; // T = state->pos + 1 ...
+    int pos_host;             // ... unless the host knows the position (>= 0): saves the kernel a dependent load
     int n_heads;
     int head_dim;
     int max_seq_len;
-    int n_splits;             // grid.y; with more than one, a second small kernel merges the partial results
+    int n_splits;             // grid.y: blocks per head, each covering an equal share of the T positions
     float *out;               // [n_heads x head_dim]
     int round_out;            // f16 rounding point before wo (transformer.rs:793-796)
-    float *workspace;         // [n_heads x n_splits x (head_dim + 2)], needed when n_splits > 1
+    float *workspace;         // [n_heads x n_splits x (head_dim + 2)] partial (max, sum, weighted V), needed when n_splits > 1
+    unsigned *tickets;        // [n_heads] arrival counters, needed when n_splits > 1 and the merge runs inside the kernel;
+                              // zero before the launch, and the kernel leaves them zero
+    int merge_mode;           // 0: a second small kernel merges the partial results; 1 / 2: the last block of a head to finish
+                              // merges them (1: device-scope fences around the ticket, 2: device-scope stores and loads)
+    int chunk_hint;           // upper bound of the positions one block covers (sizes the loads in flight); 0 = unknown
+    int lds_stage;            // 1: K / V tiles staged in LDS first (comparison variant; needs pos_host, an f16 cache, head_dim 64 / 128)
 };
 
 hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s);
+size_t attn_decode_workspace_floats(int n_heads, int head_dim, int n_splits);
+constexpr int kAttnDecodeMaxSplits = 64;
 
 // ---- prefill: C = A * B^T on the matrix cores (gemm.hip) ----
 enum GemmEpilogue {
@@ -163,10 +172,10 @@ hipError_t launch_rope_kv_prefill(const PrefillRopeParams &p, hipStream_t s);
 hipError_t launch_causal_softmax(const float *scores, void *p_hi, void *p_lo, int n_heads, int n, int t_pad, int p_stride, int head_dim, hipStream_t s);
 
 hipError_t launch_embed(const void *table, int table_f16, int dim, const DecodeState *state, float *x, hipStream_t s);
-// argmax with TokenSampler's top_k = 1 behaviour (token_sampler.rs:112-147); writes state->token, appends to
-// out_tokens[state->n_out++] and advances state->pos.
+// TokenSampler::sample at top_k = 1 (token_sampler.rs:99-147) on logits * scale (scale = 1 / temperature); writes
+// state->token, appends to out_tokens[state->n_out++] and advances state->pos.
 hipError_t launch_argmax_advance(const float *logits, int vocab, DecodeState *state, int32_t *out_tokens, int out_cap,
-                                 hipStream_t s);
+                                 hipStream_t s, float scale = 1.0f);
 hipError_t launch_set_state(DecodeState *state, int pos, int token, int reset_out, hipStream_t s);
 hipError_t launch_reset_out(DecodeState *state, hipStream_t s);
 hipError_t launch_advance_pos(DecodeState *state, const int32_t *tokens_dev, int idx, hipStream_t s);
@@ -184,6 +193,10 @@ hipError_t launch_silu(void *dst, uint64_t n, int is_f16, hipStream_t s);
 hipError_t launch_add_f32(float *dst, const float *a, const float *b, uint64_t n, hipStream_t s); // dst = a + b
 hipError_t launch_rmsnorm_rows(float *y, const float *x, const float *w, int rows, int d, float eps, int round_y, hipStream_t s);
 hipError_t launch_rope_row(float *x, int n_heads, int head_dim, const float2 *freqs_at_pos, hipStream_t s);
+hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s); // m = f16(silu(g) * u)
+// RoPE on q (in place) and k at `pos`, k and v into the cache planes [head][position][head_dim] at `pos`
+hipError_t launch_rope_kvwrite(float *q, const float *k, const float *v, void *cache_k, void *cache_v, int cache_f16, int n_heads, int head_dim,
+                               int max_seq_len, int pos, const float2 *freqs_at_pos, hipStream_t s);
 // KV-cache services (transformer.rs:180-197): shift positions left by `shifts` within each (head) plane
 hipError_t launch_cache_shift_left(void *cache, int is_f16, size_t planes, int max_seq_len, int head_dim, int shifts, hipStream_t s);
 // test hook: [head_dim x max_seq_len] f32 view of one head's plane

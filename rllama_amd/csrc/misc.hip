@@ -30,18 +30,34 @@ hipError_t launch_embed(const void *table, int table_f16, int dim, const DecodeS
 }
 
 __global__ __launch_bounds__(1024) void argmax_advance_kernel(const float *logits, int vocab, DecodeState *state,
-                                                              int32_t *out_tokens, int out_cap) {
+                                                              int32_t *out_tokens, int out_cap, float scale) {
     // TokenSampler::sample at top_k = 1 (token_sampler.rs:99-147): the max/shift loops run over
     // 0..logits.rows() == 0..1 on the transposed 1 x vocab tensor, so token 0's logit becomes l0 - l0
-    // and the rest are untouched; softmax is monotonic, so the winner is the largest shifted logit.
-    // NaN never wins (sorted last, :131-145); equal values resolve to the lowest id.
+    // and the rest are untouched; then softmax WITHOUT a maximum subtracted (tensor.rs:479-494), a sort by
+    // descending probability with NaN last (:131-145), and the first entry wins.
+    //   * While sum(exp(l)) is finite, exp and the division by the sum keep the order of the logits, so the winner is
+    //     the largest shifted logit (equal values: the lowest id).
+    //   * Once that sum is not finite every probability is 0 or NaN: a logit above ln(FLT_MAX) gives inf / inf = NaN,
+    //     everything else x / inf = 0, and a NaN logit turns the sum and with it every probability into NaN.  What wins then
+    //     is the lowest id whose probability is not NaN -- token 0, whose shifted logit is exactly 0 -- or, with every
+    //     probability NaN, the id the reference's fall-through returns, 0 as well.
+    // `scale` is 1 / temperature (:99-102; 1.0 leaves the logits as they are).
+    // The sum is only evaluated when it can overflow at all (largest logit above ln(FLT_MAX / vocab)); it is then formed in
+    // double, which decides like the reference's sequential f32 sum except within rounding of FLT_MAX itself.
     __shared__ float sval[16];
     __shared__ int sidx[16];
+    __shared__ int snan[16];
+    __shared__ double ssum[16];
+    __shared__ float s_best;
+    __shared__ int s_nan;
     const int tid = threadIdx.x;
     float best = -INFINITY;
     int besti = -1;
+    int seen_nan = 0;
     auto consider = [&](float v, int i) {
+        v = v * scale;
         if (i == 0) v = v - v;
+        if (v != v) seen_nan = 1;
         if (v > best || (besti < 0 && v == best)) {
             best = v;
             besti = i;
@@ -75,6 +91,7 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const float *logit
     for (int off = 32; off >= 1; off >>= 1) {
         float ov = __shfl_xor(best, off, kWave);
         int oi = __shfl_xor(besti, off, kWave);
+        seen_nan |= __shfl_xor(seen_nan, off, kWave);
         bool take = (oi >= 0) && (besti < 0 || ov > best || (ov == best && oi < besti));
         if (take) {
             best = ov;
@@ -82,23 +99,48 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const float *logit
         }
     }
     const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int nw = blockDim.x / kWave;
     if (lane == 0) {
         sval[wave] = best;
         sidx[wave] = besti;
+        snan[wave] = seen_nan;
     }
     __syncthreads();
     if (tid == 0) {
-        const int nw = blockDim.x / kWave;
         for (int w = 1; w < nw; w++) {
             float ov = sval[w];
             int oi = sidx[w];
+            seen_nan |= snan[w];
             bool take = (oi >= 0) && (besti < 0 || ov > best || (ov == best && oi < besti));
             if (take) {
                 best = ov;
                 besti = oi;
             }
         }
-        if (besti < 0) besti = 0; // every logit NaN
+        s_best = best;
+        s_nan = seen_nan;
+    }
+    __syncthreads();
+    // can sum(exp(l)) overflow f32?  Only if vocab * exp(largest) can: largest > ln(FLT_MAX) - ln(vocab)
+    const float kLnFltMax = 88.72283172607422f; // expf overflows above this value
+    const bool sum_at_risk = !s_nan && s_best <= kLnFltMax && s_best > kLnFltMax - logf((float)vocab);
+    double total = 0.0;
+    if (sum_at_risk) { // block-uniform
+        double part = 0.0;
+        for (int i = tid; i < vocab; i += blockDim.x) {
+            const float v = i == 0 ? 0.0f : logits[i] * scale;
+            part += exp((double)v);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) part += __shfl_xor(part, off, kWave);
+        if (lane == 0) ssum[wave] = part;
+        __syncthreads();
+        if (tid == 0)
+            for (int w = 0; w < nw; w++) total += ssum[w];
+    }
+    if (tid == 0) {
+        if (besti < 0) besti = 0;                                           // every logit NaN
+        if (seen_nan || best > kLnFltMax || total > 3.4028234663852886e38) besti = 0; // sum not finite: see above
         state->token = besti;
         state->pos = state->pos + 1;
         const int k = state->n_out;
@@ -108,8 +150,8 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const float *logit
 }
 
 hipError_t launch_argmax_advance(const float *logits, int vocab, DecodeState *state, int32_t *out_tokens, int out_cap,
-                                 hipStream_t s) {
-    hipLaunchKernelGGL(argmax_advance_kernel, dim3(1), dim3(1024), 0, s, logits, vocab, state, out_tokens, out_cap);
+                                 hipStream_t s, float scale) {
+    hipLaunchKernelGGL(argmax_advance_kernel, dim3(1), dim3(1024), 0, s, logits, vocab, state, out_tokens, out_cap, scale);
     return hipGetLastError();
 }
 
@@ -310,6 +352,55 @@ __global__ void rope_row_kernel(float *x, int n_heads, int head_dim, const float
 hipError_t launch_rope_row(float *x, int n_heads, int head_dim, const float2 *freqs_at_pos, hipStream_t s) {
     const int total = n_heads * (head_dim / 2);
     hipLaunchKernelGGL(rope_row_kernel, dim3((total + 255) / 256), dim3(256), 0, s, x, n_heads, head_dim, freqs_at_pos);
+    return hipGetLastError();
+}
+
+// m = silu(g) * u on f16 tensors: g and u are f16 values (projection outputs, tensor.rs:1623-1643), the product is formed
+// in f32 and rounded once (transformer.rs:557-565)
+__global__ void silu_mul_f16_kernel(const half_t *g, const half_t *u, half_t *m, size_t total) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const float x = (float)g[i];
+        m[i] = (half_t)((x / (1.0f + expf(-x))) * (float)u[i]);
+    }
+}
+
+hipError_t launch_silu_mul_f16(const void *g, const void *u, void *m, size_t total, hipStream_t s) {
+    hipLaunchKernelGGL(silu_mul_f16_kernel, dim3(fill_blocks(total)), dim3(256), 0, s, (const half_t *)g, (const half_t *)u, (half_t *)m, total);
+    return hipGetLastError();
+}
+
+// One token's attention inputs (transformer.rs:704-761 with seq_len 1): RoPE on q (in place) and on k, then k and v go
+// into the cache planes [head][position][head_dim] at `pos`, rounded to f16 where the cache is f16.
+template <typename CT>
+__global__ void rope_kvwrite_kernel(float *q, const float *k, const float *v, CT *cache_k, CT *cache_v, int n_heads, int head_dim, int max_seq_len,
+                                    int pos, const float2 *freqs) {
+    const int half = head_dim / 2;
+    const int total = n_heads * half;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        const int h = i / half, c = i - h * half;
+        const size_t e = (size_t)h * head_dim + 2 * c;
+        float a, b;
+        rope_pair(q[e], q[e + 1], freqs[c], a, b);
+        q[e] = a;
+        q[e + 1] = b;
+        rope_pair(k[e], k[e + 1], freqs[c], a, b);
+        const size_t idx = ((size_t)h * max_seq_len + pos) * head_dim + 2 * c;
+        cache_k[idx] = (CT)a; // Tensor::set_f32 on the cache's dtype (tensor.rs:373-376)
+        cache_k[idx + 1] = (CT)b;
+        cache_v[idx] = (CT)v[e];
+        cache_v[idx + 1] = (CT)v[e + 1];
+    }
+}
+
+hipError_t launch_rope_kvwrite(float *q, const float *k, const float *v, void *cache_k, void *cache_v, int cache_f16, int n_heads, int head_dim,
+                               int max_seq_len, int pos, const float2 *freqs_at_pos, hipStream_t s) {
+    const int total = n_heads * (head_dim / 2);
+    dim3 g((total + 255) / 256), b(256);
+    if (cache_f16)
+        hipLaunchKernelGGL(rope_kvwrite_kernel<half_t>, g, b, 0, s, q, k, v, (half_t *)cache_k, (half_t *)cache_v, n_heads, head_dim, max_seq_len, pos, freqs_at_pos);
+    else
+        hipLaunchKernelGGL(rope_kvwrite_kernel<float>, g, b, 0, s, q, k, v, (float *)cache_k, (float *)cache_v, n_heads, head_dim, max_seq_len, pos, freqs_at_pos);
     return hipGetLastError();
 }
 

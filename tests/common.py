@@ -152,3 +152,29 @@ class RefF64:
             x = h_ + self.r(mm @ W[(W2, l)].T)
         xf = self.norm(x, W[(NORM, 0)])
         return xf[-1] @ W[(OUTPUT, 0)].T
+
+
+def oracle_from_device(gm: "rllama_amd.Transformer", max_seq_len: int) -> oracle.Model:
+    """An oracle model holding exactly the bits the device model holds (f16 mode): every tensor is read back from HBM and
+    handed to the oracle, so both sides start from the same weights whatever filled them."""
+    d, L, H, F, V = gm.dim, gm.n_layers, gm.n_heads, gm.ffn_hidden, gm.vocab_size
+    om = oracle.Model(d, L, H, F, V, max_seq_len, gm.params.norm_eps, True)
+    shapes = {WQ: (d, d), WK: (d, d), WV: (d, d), WO: (d, d), W1: (F, d), W3: (F, d), W2: (d, F)}
+    for kind in (TOK_EMB, OUTPUT):
+        om.set_tensor(kind, 0, gm.get_tensor(kind, 0, V, d, as_f16_bits=True))
+    om.set_tensor(NORM, 0, gm.get_tensor(NORM, 0, 1, d))
+    for l in range(L):
+        for kind, (r, c) in shapes.items():
+            om.set_tensor(kind, l, gm.get_tensor(kind, l, r, c, as_f16_bits=True))
+        for kind in (ATTN_NORM, FFN_NORM):
+            om.set_tensor(kind, l, gm.get_tensor(kind, l, 1, d))
+    return om
+
+
+def elementwise_rel_err(a: np.ndarray, b: np.ndarray, floor_frac: float = 0.01) -> float:
+    """max |a - b| / |b| over the entries with |b| above floor_frac of the largest |b| (an element-wise relative error that
+    leaves out the entries small through cancellation)."""
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    keep = np.abs(b) >= floor_frac * np.max(np.abs(b))
+    return float(np.max(np.abs(a - b)[keep] / np.abs(b)[keep]))

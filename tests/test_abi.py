@@ -31,6 +31,33 @@ def test_library_exports_every_declared_symbol():
     assert lib.rlh_abi_version() == 1
 
 
+def test_rust_ffi_crate_matches_the_header():
+    """rust/rllama-hip-sys/src/lib.rs (the extern "C" seam a Rust host links against) is what the generator makes of the
+    header today, and declares every function with the argument count of the ctypes table."""
+    import importlib.util
+    root = os.path.dirname(HERE)
+    gen_path = os.path.join(root, "rust", "rllama-hip-sys", "gen_bindings.py")
+    spec = importlib.util.spec_from_file_location("gen_bindings", gen_path)
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    lib_rs = open(os.path.join(root, "rust", "rllama-hip-sys", "src", "lib.rs")).read()
+    assert lib_rs == gen.generate(), "run `python rust/rllama-hip-sys/gen_bindings.py` after changing include/rllama_hip.h"
+    decls = dict((m.group(1), m.group(2)) for m in re.finditer(r"pub fn (rlh_[a-z0-9_]+)\((.*?)\)(?: -> [^;]+)?;", lib_rs))
+    assert sorted(decls) == _declared_symbols()
+    for name, (res, args) in _lib.SIGNATURES.items():
+        n_rust = 0 if not decls[name].strip() else decls[name].count(":")
+        assert n_rust == len(args), (name, decls[name])
+    for const in ("RLH_OK", "RLH_ERR_UNSUPPORTED", "RLH_F16", "RLH_F32", "RLH_TOK_EMB", "RLH_OUTPUT"):
+        assert f"pub const {const}: c_int" in lib_rs
+    for field in [f[0] for f in _lib.ModelParams._fields_] + [f[0] for f in _lib.SamplerParams._fields_]:
+        assert f"pub {field}:" in lib_rs
+    # what INTEGRATION.md shows of the seam must exist in the crate
+    doc = open(os.path.join(root, "INTEGRATION.md")).read()
+    for name in set(re.findall(r"\b(rlh_[a-z0-9_]+)\b", doc)):
+        assert name in decls or name in ("rlh_model_params", "rlh_sampler_params", "rlh_ctx", "rlh_model", "rlh_caches", "rlh_tensor", "rlh_event",
+                                         "rlh_tensor_kind", "rlh_status", "rlh_dtype"), f"INTEGRATION.md names {name}, which the header does not declare"
+
+
 def test_no_oracle_in_product():
     """The shipped package and library must not reach into oracle/ (test infrastructure)."""
     pkg = os.path.dirname(_lib.__file__)
