@@ -138,6 +138,22 @@ void orc_f16_to_f32_array(const uint16_t *src, float *dst, size_t n) {
 /* dot8 and friends                                                                            */
 /* ------------------------------------------------------------------------------------------ */
 
+/* Sensitivity probe, off by default (orc_set_alt_order): with it on, the f16 projections sum their products in another,
+ * equally valid fp32 order -- two sets of 8 lanes taking alternate blocks of 8, joined at the end, and the horizontal sum
+ * taken left to right.  The values this produces are NOT the reference's; the switch exists to measure how far the
+ * reference's own arithmetic moves under a reordering of its additions (the distance any other implementation can be
+ * expected to stay within). */
+static int g_alt_order = 0;
+void orc_set_alt_order(int on) { g_alt_order = on ? 1 : 0; }
+
+static inline float hsum8_alt(__m256 ymm) {
+    float l[8];
+    _mm256_storeu_ps(l, ymm);
+    float t = l[0];
+    for (int i = 1; i < 8; i++) t += l[i];
+    return t;
+}
+
 static inline float hsum8_v(__m256 ymm) {
     /* simd_support.rs:97-105, instruction for instruction */
     __m256 ymm2 = _mm256_permute2f128_ps(ymm, ymm, 1);
@@ -208,6 +224,33 @@ static inline void dot8x4_f16(const uint16_t *x, const uint16_t *w0, const uint1
                               const uint16_t *w3, int k, float out[4]) {
     __m256 a0 = _mm256_setzero_ps(), a1 = a0, a2 = a0, a3 = a0;
     int p = 0;
+    if (g_alt_order) { /* not the reference's order: see orc_set_alt_order */
+        __m256 b0 = a0, b1 = a0, b2 = a0, b3 = a0;
+        for (; p + 16 <= k; p += 16) {
+            __m256 xv = load8_f16(x + p), xw = load8_f16(x + p + 8);
+            a0 = _mm256_fmadd_ps(xv, load8_f16(w0 + p), a0);
+            a1 = _mm256_fmadd_ps(xv, load8_f16(w1 + p), a1);
+            a2 = _mm256_fmadd_ps(xv, load8_f16(w2 + p), a2);
+            a3 = _mm256_fmadd_ps(xv, load8_f16(w3 + p), a3);
+            b0 = _mm256_fmadd_ps(xw, load8_f16(w0 + p + 8), b0);
+            b1 = _mm256_fmadd_ps(xw, load8_f16(w1 + p + 8), b1);
+            b2 = _mm256_fmadd_ps(xw, load8_f16(w2 + p + 8), b2);
+            b3 = _mm256_fmadd_ps(xw, load8_f16(w3 + p + 8), b3);
+        }
+        for (; p < k; p++) { /* leftovers one by one into lane 0 */
+            float xs = orc_f16_bits_to_f32(x[p]);
+            float t[8] = {0};
+            t[0] = xs * orc_f16_bits_to_f32(w0[p]); a0 = _mm256_add_ps(a0, _mm256_loadu_ps(t));
+            t[0] = xs * orc_f16_bits_to_f32(w1[p]); a1 = _mm256_add_ps(a1, _mm256_loadu_ps(t));
+            t[0] = xs * orc_f16_bits_to_f32(w2[p]); a2 = _mm256_add_ps(a2, _mm256_loadu_ps(t));
+            t[0] = xs * orc_f16_bits_to_f32(w3[p]); a3 = _mm256_add_ps(a3, _mm256_loadu_ps(t));
+        }
+        out[0] = hsum8_alt(_mm256_add_ps(a0, b0));
+        out[1] = hsum8_alt(_mm256_add_ps(a1, b1));
+        out[2] = hsum8_alt(_mm256_add_ps(a2, b2));
+        out[3] = hsum8_alt(_mm256_add_ps(a3, b3));
+        return;
+    }
     for (; p + 8 <= k; p += 8) {
         __m256 xv = load8_f16(x + p);
         a0 = _mm256_fmadd_ps(xv, load8_f16(w0 + p), a0);

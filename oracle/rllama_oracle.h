@@ -117,6 +117,9 @@ void orc_set_threads(int n);   /* rayon pool size analogue (rllama_main.rs:148-1
 int  orc_get_threads(void);
 /* 1: one-row f32 products (output head; w1/w2/w3 in f32 mode) run on one thread like tensor.rs:1837-1918. Timing only. */
 void orc_set_reference_threading(int on);
+/* Sensitivity probe (default off): the f16 projections sum their products in another valid fp32 order (not the reference's).
+ * Measures how far the reference's own results move under a reordering of its additions. */
+void orc_set_alt_order(int on);
 
 orc_model *orc_model_create(const orc_params *p);
 void       orc_model_free(orc_model *m);

@@ -107,6 +107,12 @@ struct rlh_model {
     int attn_chunk = 128;      // positions per block beyond that
     int attn_merge_mode = 2;   // how the blocks of a split sequence are merged (AttnDecodeParams::merge_mode)
     bool capturing = false;    // a decode step is being recorded into a HIP graph
+    // fused layer kernel (decode_fused.hip), RLLAMA_HIP_FUSED=1; otherwise one launch per matrix-vector product
+    bool fused_layers = getenv("RLLAMA_HIP_FUSED") && atoi(getenv("RLLAMA_HIP_FUSED")) != 0;
+    FusedBarrierState *fused_barrier = nullptr;
+    long long fused_limit_ticks = 20000000; // 200 ms at the 100 MHz wall clock
+    int fused_blocks[4] = {0, 0, 0, 0};     // grid per kernel variant (last phase wq|wk|wv / f16 head / f32 head / none), 0 = not yet asked
+    bool fused_used = false;                // a fused kernel was enqueued since the error word was last checked
     bool attn_lds_stage = getenv("RLLAMA_HIP_ATTN_LDS") && atoi(getenv("RLLAMA_HIP_ATTN_LDS")) != 0; // comparison variant of the decode attention
     int stream_weights = 1;
     PrefillScratch pf;
@@ -330,6 +336,7 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     B((void **)&m->prompt_dev, sizeof(int32_t) * m->prompt_cap);
     B((void **)&m->attn_ws, sizeof(float) * attn_decode_workspace_floats(prm->n_heads, hd, m->max_splits));
     B((void **)&m->attn_tickets, sizeof(unsigned) * (size_t)prm->n_heads);
+    B((void **)&m->fused_barrier, sizeof(FusedBarrierState));
     if (rc == RLH_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(RLH_ERR_HIP, "rlh_model_create: hipDeviceSynchronize failed");
     if (rc != RLH_OK) {
         rlh_model_free(m);
@@ -356,7 +363,7 @@ extern "C" void rlh_model_free(rlh_model *m) {
     free_weight(m->norm);
     free_weight(m->output);
     m->pf.release();
-    void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws, m->attn_tickets};
+    void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws, m->attn_tickets, m->fused_barrier};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -650,10 +657,9 @@ static int attn_splits(const rlh_model *m, int T) { return attn_splits_rule(T, m
 
 enum StepKernel { kStepQkv = 0, kStepAttn = 1, kStepWo = 2, kStepW13 = 3, kStepW2 = 4, kStepHead = 5 };
 
-// Enqueues one of the five kernels of layer l (or the output head) for the token described by the device
-// state.  T_host = position + 1 as known to the host (sizes the attention grid).
-static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, int T_host, int first_layer = 0) {
-    hipStream_t st = m->ctx->stream;
+// The launch parameters of one matrix-vector kernel of layer l (or of the output head) for the token described by the
+// device state; *epi receives its epilogue.  which: kStepQkv, kStepWo, kStepW13, kStepW2, kStepHead.
+static void build_gemv_step(rlh_model *m, rlh_caches *c, int l, int which, int first_layer, GemvParams *out, int *epi) {
     const rlh_model_params &P = m->prm;
     const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size;
     const int f16 = P.force_f16 ? 1 : 0;
@@ -682,19 +688,18 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         p.y = m->logits;
         p.n_rows = V;
         p.k = d;
-        HIP_TRY(launch_gemv(p, kEpiStore, st));
-        return RLH_OK;
+        *out = p;
+        *epi = kEpiStore;
+        return;
     }
     Layer &L = m->layers[(size_t)l];
-    const size_t layer_elems = (size_t)P.n_heads * P.max_seq_len * m->head_dim;
-    const size_t ces = c->f16 ? 2 : 4;
-    void *ck = (char *)c->k + (size_t)l * layer_elems * ces;
-    void *cv = (char *)c->v + (size_t)l * layer_elems * ces;
+    GemvParams p = g;
     switch (which) {
     case kStepQkv: {
         // (previous layer's second residual add, transformer.rs:445) + attention_norm + wq|wk|wv + RoPE + cache
         // write (transformer.rs:432, 665-668, 694-725, 751-761)
-        GemvParams p = g;
+        const size_t layer_elems = (size_t)P.n_heads * P.max_seq_len * m->head_dim;
+        const size_t ces = c->f16 ? 2 : 4;
         p.w = L.wqkv.p;
         if (l == first_layer) {
             p.x = m->x;
@@ -709,53 +714,26 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         p.k = d;
         p.state = m->state;
         p.freqs = m->freqs;
-        p.cache_k = ck;
-        p.cache_v = cv;
+        p.cache_k = (char *)c->k + (size_t)l * layer_elems * ces;
+        p.cache_v = (char *)c->v + (size_t)l * layer_elems * ces;
         p.cache_f16 = c->f16;
         p.dim = d;
         p.head_dim = m->head_dim;
         p.max_seq_len = P.max_seq_len;
-        HIP_TRY(launch_gemv(p, kEpiRopeKv, st));
+        *epi = kEpiRopeKv;
         break;
     }
-    case kStepAttn: {
-        // scores, softmax, P.V (transformer.rs:762-779) + f16 rounding point before wo (:793-796)
-        AttnDecodeParams a{};
-        a.q = m->q;
-        a.cache_k = ck;
-        a.cache_v = cv;
-        a.cache_f16 = c->f16;
-        a.state = m->state;
-        a.pos_host = m->capturing ? -1 : T_host - 1; // a captured step is replayed at later positions: it reads the device state
-        a.n_heads = P.n_heads;
-        a.head_dim = m->head_dim;
-        a.max_seq_len = P.max_seq_len;
-        a.n_splits = attn_splits(m, T_host);
-        a.out = m->att;
-        a.round_out = f16;
-        a.workspace = m->attn_ws;
-        a.tickets = m->attn_tickets;
-        a.merge_mode = m->attn_merge_mode;
-        a.chunk_hint = (((T_host + a.n_splits - 1) / a.n_splits) + 15) & ~15;
-        a.lds_stage = m->attn_lds_stage && !m->capturing && c->f16 && (m->head_dim == 128 || m->head_dim == 64) && a.merge_mode == 2 &&
-                      (size_t)a.chunk_hint * m->head_dim * 4 <= 128 * 1024;
-        HIP_TRY(launch_attn_decode(a, st));
-        break;
-    }
-    case kStepWo: {
+    case kStepWo:
         // wo (transformer.rs:783-819); its output joins the stream in the next kernel
-        GemvParams p = g;
         p.w = L.wo.p;
         p.x = m->att;
         p.y = m->att_o;
         p.n_rows = d;
         p.k = d;
-        HIP_TRY(launch_gemv(p, kEpiStore, st));
+        *epi = kEpiStore;
         break;
-    }
-    case kStepW13: {
+    case kStepW13:
         // h = x + att_out (transformer.rs:442) + ffn_norm + w1|w3 + SiLU * gate (transformer.rs:443, 537-565)
-        GemvParams p = g;
         p.w = L.w1.p;
         p.w_b = L.w3.p;
         p.x = m->x;
@@ -765,29 +743,118 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         p.y = m->mh;
         p.n_rows = F;
         p.k = d;
-        HIP_TRY(launch_gemv(p, kEpiSilu, st));
+        *epi = kEpiSilu;
         break;
-    }
-    case kStepW2: {
+    default: // kStepW2
         // w2 (transformer.rs:568-570); its output joins the stream in the next kernel
-        GemvParams p = g;
         p.w = L.w2.p;
         p.x = m->mh;
         p.y = m->ffn_o;
         p.n_rows = d;
         p.k = F;
-        HIP_TRY(launch_gemv(p, kEpiStore, st));
+        *epi = kEpiStore;
         break;
     }
-    default: return fail(RLH_ERR_INVALID, "unknown step kernel %d", which);
+    *out = p;
+}
+
+// Enqueues one of the five kernels of layer l (or the output head) for the token described by the device
+// state.  T_host = position + 1 as known to the host (sizes the attention grid).
+static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, int T_host, int first_layer = 0) {
+    hipStream_t st = m->ctx->stream;
+    const rlh_model_params &P = m->prm;
+    if (which < kStepQkv || which > kStepHead) return fail(RLH_ERR_INVALID, "unknown step kernel %d", which);
+    if (which != kStepAttn) {
+        GemvParams p;
+        int epi = kEpiStore;
+        build_gemv_step(m, c, l, which, first_layer, &p, &epi);
+        HIP_TRY(launch_gemv(p, epi, st));
+        return RLH_OK;
     }
+    // scores, softmax, P.V (transformer.rs:762-779) + f16 rounding point before wo (:793-796)
+    const size_t layer_elems = (size_t)P.n_heads * P.max_seq_len * m->head_dim;
+    const size_t ces = c->f16 ? 2 : 4;
+    AttnDecodeParams a{};
+    a.q = m->q;
+    a.cache_k = (char *)c->k + (size_t)l * layer_elems * ces;
+    a.cache_v = (char *)c->v + (size_t)l * layer_elems * ces;
+    a.cache_f16 = c->f16;
+    a.state = m->state;
+    a.pos_host = m->capturing ? -1 : T_host - 1; // a captured step is replayed at later positions: it reads the device state
+    a.n_heads = P.n_heads;
+    a.head_dim = m->head_dim;
+    a.max_seq_len = P.max_seq_len;
+    a.n_splits = attn_splits(m, T_host);
+    a.out = m->att;
+    a.round_out = P.force_f16 ? 1 : 0;
+    a.workspace = m->attn_ws;
+    a.tickets = m->attn_tickets;
+    a.merge_mode = m->attn_merge_mode;
+    a.chunk_hint = (((T_host + a.n_splits - 1) / a.n_splits) + 15) & ~15;
+    a.lds_stage = m->attn_lds_stage && !m->capturing && c->f16 && (m->head_dim == 128 || m->head_dim == 64) && a.merge_mode == 2 &&
+                  (size_t)a.chunk_hint * m->head_dim * 4 <= 128 * 1024;
+    HIP_TRY(launch_attn_decode(a, st));
     return RLH_OK;
+}
+
+// The matrix-vector kernels of layer l after its attention -- wo, w1|w3, w2 -- and what follows them (the next layer's
+// wq|wk|wv, or the output head after the last layer when with_head is set) as one launch (decode_fused.hip).
+static int enqueue_fused_layer(rlh_model *m, rlh_caches *c, int l, bool with_head) {
+    FusedLayerParams F{};
+    int epi = 0;
+    build_gemv_step(m, c, l, kStepWo, 0, &F.wo, &epi);
+    build_gemv_step(m, c, l, kStepW13, 0, &F.w13, &epi);
+    build_gemv_step(m, c, l, kStepW2, 0, &F.w2, &epi);
+    const bool last_layer = l + 1 == m->prm.n_layers;
+    F.n_phases = 4;
+    if (!last_layer) {
+        build_gemv_step(m, c, l + 1, kStepQkv, 0, &F.last, &epi);
+        F.last_kind = 0;
+    } else if (with_head) {
+        build_gemv_step(m, c, 0, kStepHead, 0, &F.last, &epi);
+        F.last_kind = m->output.f16 ? 1 : 2;
+    } else {
+        F.n_phases = 3;
+        F.last_kind = 0;
+    }
+    F.barrier = m->fused_barrier;
+    F.limit_ticks = m->fused_limit_ticks;
+    int &blocks = m->fused_blocks[F.n_phases == 3 ? 3 : F.last_kind];
+    if (blocks == 0) HIP_TRY(fused_layer_grid(F, m->ctx->prop.multiProcessorCount, &blocks));
+    HIP_TRY(launch_fused_layer(F, blocks, m->ctx->stream));
+    m->fused_used = true;
+    return RLH_OK;
+}
+
+// After the work of a call has completed: did a device-wide barrier of the fused kernel give up?  Then the results of the
+// call are void; the barrier words are cleared so that later calls start clean.
+static int check_fused_barrier(rlh_model *m) {
+    if (!m->fused_used) return RLH_OK;
+    m->fused_used = false;
+    unsigned err = 0;
+    const size_t err_off = sizeof(unsigned) * (size_t)(kFusedGroups + 2) * 32;
+    HIP_TRY(hipMemcpy(&err, (const char *)m->fused_barrier + err_off, sizeof(err), hipMemcpyDeviceToHost));
+    if (err == 0) return RLH_OK;
+    HIP_TRY(hipMemset(m->fused_barrier, 0, sizeof(FusedBarrierState)));
+    m->next_pos = -1;
+    m->greedy_caches = nullptr;
+    return fail(RLH_ERR_HIP, "a device-wide barrier of the fused layer kernel did not complete within its time limit (not every workgroup "
+                             "was resident: is another process using the device?); the call's results are void");
 }
 
 // Enqueues one token step (the body of Transformer::forward for a single row, transformer.rs:361-381):
 // reads state->token / state->pos on the device.
 static int enqueue_token_step(rlh_model *m, rlh_caches *c, int T_host, bool with_head) {
     HIP_TRY(launch_embed(m->tok_emb.p, m->tok_emb.f16, m->prm.dim, m->state, m->x, m->ctx->stream));
+    if (m->fused_layers) {
+        // wq|wk|wv of layer 0 alone, then per layer: attention, and one launch for everything up to the next attention
+        int rc = enqueue_step_kernel(m, c, 0, kStepQkv, T_host);
+        for (int l = 0; rc == RLH_OK && l < m->prm.n_layers; l++) {
+            rc = enqueue_step_kernel(m, c, l, kStepAttn, T_host);
+            if (rc == RLH_OK) rc = enqueue_fused_layer(m, c, l, with_head);
+        }
+        return rc;
+    }
     for (int l = 0; l < m->prm.n_layers; l++) {
         for (int which = kStepQkv; which <= kStepW2; which++) {
             int rc = enqueue_step_kernel(m, c, l, which, T_host);

@@ -1,0 +1,407 @@
+// gemv_device.h -- device code of the batch-1 decode GEMV (gemv.hip has the design notes), shared by the stand-alone
+// kernel (gemv.hip) and the fused layer kernel (decode_fused.hip).
+#pragma once
+
+#include "kernels.h"
+#include "device_utils.h"
+
+namespace rlh {
+
+// Launch shape (overridable at compile time for tuning runs).
+#ifndef RLH_GEMV_WAVES
+#define RLH_GEMV_WAVES 4
+#endif
+#ifndef RLH_GEMV_TARGET_WAVES
+#define RLH_GEMV_TARGET_WAVES 2048 // 256 CUs x 8 resident wavefronts
+#endif
+#ifndef RLH_GEMV_BURST
+#define RLH_GEMV_BURST 8
+#endif
+constexpr int kGemvWaves = RLH_GEMV_WAVES;
+constexpr int kGemvThreads = kGemvWaves * kWave;
+constexpr int kGemvTargetWaves = RLH_GEMV_TARGET_WAVES;
+constexpr int kGemvBurst = RLH_GEMV_BURST; // 16-byte loads per lane issued back to back before they are consumed
+#ifndef RLH_GEMV_PRELOAD
+#define RLH_GEMV_PRELOAD 1
+#endif
+#ifndef RLH_GEMV_PROLOGUE_VECS
+#define RLH_GEMV_PROLOGUE_VECS 8
+#endif
+constexpr int kGemvPrologueVecs = RLH_GEMV_PROLOGUE_VECS; // float4 loads per thread per prologue batch (one batch covers k <= 1024 * this)
+
+template <typename WT>
+struct WVec;
+template <>
+struct WVec<half_t> {
+    static constexpr int kVec = 8;
+    __device__ static __forceinline__ void unpack(const uint4_t &raw, float (&out)[8]) {
+        half8_t h = __builtin_bit_cast(half8_t, raw);
+#pragma unroll
+        for (int i = 0; i < 8; i++) out[i] = (float)h[i];
+    }
+};
+template <>
+struct WVec<float> {
+    static constexpr int kVec = 4;
+    __device__ static __forceinline__ void unpack(const uint4_t &raw, float (&out)[4]) {
+        float4_t f = __builtin_bit_cast(float4_t, raw);
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = f[i];
+    }
+};
+
+template <typename XT, int kVec>
+__device__ __forceinline__ void load_x(const XT *xs, float (&out)[kVec]) {
+    if constexpr (sizeof(XT) == 2 && kVec == 8) {
+        half8_t h = *reinterpret_cast<const half8_t *>(xs);
+#pragma unroll
+        for (int i = 0; i < 8; i++) out[i] = (float)h[i];
+    } else if constexpr (sizeof(XT) == 2 && kVec == 4) {
+        typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
+        half4_t h = *reinterpret_cast<const half4_t *>(xs);
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = (float)h[i];
+    } else if constexpr (sizeof(XT) == 4 && kVec == 8) {
+        float4_t a = *reinterpret_cast<const float4_t *>(xs);
+        float4_t b = *reinterpret_cast<const float4_t *>(xs + 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            out[i] = a[i];
+            out[i + 4] = b[i];
+        }
+    } else {
+        float4_t a = *reinterpret_cast<const float4_t *>(xs);
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = a[i];
+    }
+}
+
+// iterations of 64 lanes x vec elements that cover k, and the LDS footprint that goes with them
+__host__ __device__ inline int gemv_iters(int k, int vec) { return (k + kWave * vec - 1) / (kWave * vec); }
+
+// Sum over the wavefront, valid in lane 63 only (no broadcast).
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+    v = group_sum<16>(v);
+    v = dpp_add<kDppRowBcast15, 0xa>(v);
+    v = dpp_add<kDppRowBcast31, 0xc>(v);
+    return v;
+}
+
+// ---- activations that cross workgroups inside one launch --------------------------------------------------------------
+// Between kernels the launch boundary makes every store visible.  Inside the fused layer kernel an activation vector is
+// written by some workgroups and read by all of them after a device-wide barrier, and the eight L2 caches of the part are
+// not coherent with each other for ordinary accesses: such vectors are therefore stored and loaded at device scope
+// (write-through stores, loads that do not take a stale L2 line).  kDev selects that form.
+template <bool kDev>
+__device__ __forceinline__ float4_t act_load4(const float4_t *p) {
+    if constexpr (kDev) {
+        const unsigned long long *q = reinterpret_cast<const unsigned long long *>(p);
+        const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float4_t v;
+        v[0] = __builtin_bit_cast(float, (unsigned)(lo & 0xffffffffull));
+        v[1] = __builtin_bit_cast(float, (unsigned)(lo >> 32));
+        v[2] = __builtin_bit_cast(float, (unsigned)(hi & 0xffffffffull));
+        v[3] = __builtin_bit_cast(float, (unsigned)(hi >> 32));
+        return v;
+    } else {
+        return *p;
+    }
+}
+template <bool kDev>
+__device__ __forceinline__ float act_load1(const float *p) {
+    if constexpr (kDev) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else return *p;
+}
+template <bool kDev>
+__device__ __forceinline__ void act_store4(float4_t *p, float4_t v) {
+    if constexpr (kDev) {
+        unsigned long long *q = reinterpret_cast<unsigned long long *>(p);
+        const unsigned long long lo = (unsigned long long)__builtin_bit_cast(unsigned, v[0]) | ((unsigned long long)__builtin_bit_cast(unsigned, v[1]) << 32);
+        const unsigned long long hi = (unsigned long long)__builtin_bit_cast(unsigned, v[2]) | ((unsigned long long)__builtin_bit_cast(unsigned, v[3]) << 32);
+        __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(q + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        *p = v;
+    }
+}
+template <bool kDev>
+__device__ __forceinline__ void act_store1(float *p, float v) {
+    if constexpr (kDev) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
+// How the first burst of the first row unit reaches the main loop.
+enum GemvPreload {
+    kPreNone = 0,   // loaded in the main loop like every other burst
+    kPreSelf = 1,   // issued by the prologue right behind its own loads (they stay ahead of it in the in-order return queue),
+                    // so that its memory latency runs under the norm / staging work
+    kPreGiven = 2   // issued by the caller before this phase began (the fused kernel issues it before the barrier it waits at)
+};
+
+template <typename WT, int kEpi>
+struct GemvShape {
+    static constexpr int kVec = WVec<WT>::kVec;
+    static constexpr int kMats = (kEpi == kEpiSilu) ? 2 : 1;    // w1 and w3 share x and the epilogue
+    static constexpr int kRows = (kEpi == kEpiRopeKv) ? 2 : 1;  // a RoPE pair (2j, 2j+1) is produced by one wave
+    static constexpr int kU = kGemvBurst / (kMats * kRows);     // pieces of one row per burst
+    static constexpr int kPiece = kWave * kVec;                  // elements one wave-wide load covers
+};
+
+// Issues the first burst of this wavefront's first row unit into wpre (kGemvBurst 16-byte loads) if that unit exists and
+// starts with a full burst; returns whether it did.  The loads do not depend on x.
+template <typename WT, int kEpi, bool kStream>
+__device__ __forceinline__ bool gemv_issue_first_burst(const GemvParams &p, uint4_t (&wpre)[kGemvBurst]) {
+    using S = GemvShape<WT, kEpi>;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int K = p.k;
+    const int unit_first = blockIdx.x * kGemvWaves + wave;
+    const bool have = unit_first < p.n_rows / S::kRows && S::kU <= K / S::kPiece;
+    if (have) {
+        const WT *wmat[2] = {reinterpret_cast<const WT *>(p.w), reinterpret_cast<const WT *>(p.w_b)};
+#pragma unroll
+        for (int u = 0; u < S::kU; u++)
+#pragma unroll
+            for (int m = 0; m < S::kMats; m++)
+#pragma unroll
+                for (int r = 0; r < S::kRows; r++)
+                    wpre[(u * S::kMats + m) * S::kRows + r] =
+                        load16<kStream>(wmat[m] + (size_t)(unit_first * S::kRows + r) * K + (size_t)u * S::kPiece + lane * S::kVec);
+    }
+    return have;
+}
+
+// One GEMV over the whole grid: prologue (x staged in LDS), main loop, epilogue.  `smem_raw` is the block's dynamic LDS
+// (gemv_lds_bytes); `red` 16 floats and `rope_f` 64 float2 of static LDS.  kDev: x / x_add are read and y / x_out written at
+// device scope (see above).  With kPre == kPreGiven, wpre holds the first burst and have_pre says whether it was issued.
+template <typename WT, typename XT, int kEpi, bool kStream, bool kDev, int kPre>
+__device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f, uint4_t (&wpre)[kGemvBurst], bool have_pre) {
+    using S = GemvShape<WT, kEpi>;
+    constexpr int kVec = S::kVec, kMats = S::kMats, kRows = S::kRows, kU = S::kU, kPiece = S::kPiece;
+    XT *xs = reinterpret_cast<XT *>(smem_raw);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int K = p.k;
+    const int pieces = gemv_iters(K, kVec);      // incl. a partial last piece
+    const int pieces_full = K / kPiece;
+    const int kpad = pieces * kPiece;
+
+    const WT *wmat[kMats];
+    wmat[0] = reinterpret_cast<const WT *>(p.w);
+    if constexpr (kMats == 2) wmat[1] = reinterpret_cast<const WT *>(p.w_b);
+    const int unit_first = blockIdx.x * kGemvWaves + wave;
+    auto preload = [&]() {
+        if constexpr (kPre == kPreSelf) have_pre = gemv_issue_first_burst<WT, kEpi, kStream>(p, wpre);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    if constexpr (kPre == kPreNone) have_pre = false;
+
+    // ---- prologue: x = (x_in [+ x_add]) [RMSNorm] [-> f16], staged in LDS, zero padded to kpad ----
+    // All global loads of a batch are issued before any is consumed (one exposed memory latency per batch).
+    const bool writes_sum = (p.x_out != nullptr) && blockIdx.x == 0;
+    const int n4 = K / 4; // k is a multiple of 4
+    const float4_t *x4 = reinterpret_cast<const float4_t *>(p.x);
+    const float4_t *a4 = reinterpret_cast<const float4_t *>(p.x_add);
+    float4_t *o4 = reinterpret_cast<float4_t *>(p.x_out);
+    for (int i = K + tid; i < kpad; i += kGemvThreads) xs[i] = (XT)0.0f;
+    if (p.norm_w != nullptr && n4 <= kGemvPrologueVecs * kGemvThreads) {
+        // RMSNorm::forward (transformer.rs:476-480): (x * rsqrt(mean(x^2) + eps)) * w, x kept in registers
+        const float4_t *w4 = reinterpret_cast<const float4_t *>(p.norm_w);
+        float4_t xv[kGemvPrologueVecs], wv[kGemvPrologueVecs];
+#pragma unroll
+        for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = act_load4<kDev>(x4 + min(tid + j * kGemvThreads, n4 - 1));
+        if (a4 != nullptr) {
+#pragma unroll
+            for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + act_load4<kDev>(a4 + min(tid + j * kGemvThreads, n4 - 1)); // transformer.rs:442 / :445
+        }
+#pragma unroll
+        for (int j = 0; j < kGemvPrologueVecs; j++) wv[j] = w4[min(tid + j * kGemvThreads, n4 - 1)];
+        __builtin_amdgcn_sched_barrier(0);
+        preload();
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kGemvPrologueVecs; j++) {
+            const int i = tid + j * kGemvThreads;
+            if (i < n4) {
+                if (writes_sum) act_store4<kDev>(o4 + i, xv[j]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) ss = fmaf(xv[j][e], xv[j][e], ss);
+            }
+        }
+        ss = block_sum(ss, red);
+        const float rs = 1.0f / sqrtf(ss / (float)K + p.eps);
+#pragma unroll
+        for (int j = 0; j < kGemvPrologueVecs; j++) {
+            const int i = tid + j * kGemvThreads;
+            if (i < n4) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) xs[i * 4 + e] = (XT)((xv[j][e] * rs) * wv[j][e]);
+            }
+        }
+    } else if (p.norm_w != nullptr) {
+        // k too large for the register path: two passes over global memory
+        preload();
+        float ss = 0.0f;
+        for (int i = tid; i < K; i += kGemvThreads) {
+            float v = act_load1<kDev>(p.x + i);
+            if (p.x_add != nullptr) v = v + act_load1<kDev>(p.x_add + i);
+            if (writes_sum) act_store1<kDev>(p.x_out + i, v);
+            ss = fmaf(v, v, ss);
+        }
+        ss = block_sum(ss, red);
+        const float rs = 1.0f / sqrtf(ss / (float)K + p.eps);
+        for (int i = tid; i < K; i += kGemvThreads) {
+            float v = act_load1<kDev>(p.x + i);
+            if (p.x_add != nullptr) v = v + act_load1<kDev>(p.x_add + i);
+            xs[i] = (XT)((v * rs) * p.norm_w[i]);
+        }
+    } else {
+        for (int base = 0; base < n4; base += kGemvPrologueVecs * kGemvThreads) {
+            float4_t xv[kGemvPrologueVecs];
+#pragma unroll
+            for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = act_load4<kDev>(x4 + min(base + tid + j * kGemvThreads, n4 - 1));
+            if (a4 != nullptr) {
+#pragma unroll
+                for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + act_load4<kDev>(a4 + min(base + tid + j * kGemvThreads, n4 - 1));
+            }
+            if (base == 0) {
+                __builtin_amdgcn_sched_barrier(0);
+                preload();
+            }
+#pragma unroll
+            for (int j = 0; j < kGemvPrologueVecs; j++) {
+                const int i = base + tid + j * kGemvThreads;
+                if (i < n4) {
+                    if (writes_sum) act_store4<kDev>(o4 + i, xv[j]);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) xs[i * 4 + e] = (XT)xv[j][e];
+                }
+            }
+        }
+    }
+    int pos = 0;
+    if constexpr (kEpi == kEpiRopeKv) {
+        pos = p.state->pos;
+        const int half_hd = p.head_dim / 2;
+        if (tid < half_hd) rope_f[tid] = p.freqs[(size_t)pos * half_hd + tid];
+    }
+    __syncthreads();
+
+    // ---- main loop: row units interleaved over all wavefronts of the grid, so that at any moment the
+    //      grid reads one dense window of the matrix ----
+    const int n_units = p.n_rows / kRows; // n_rows is a multiple of kRows (checked on the host)
+    const int W = gridDim.x * kGemvWaves;
+
+    for (int unit = unit_first; unit < n_units; unit += W) {
+        const int row0 = unit * kRows;
+        float acc[kMats][kRows];
+#pragma unroll
+        for (int m = 0; m < kMats; m++)
+#pragma unroll
+            for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
+
+        for (int c = 0; c < pieces; c += kU) {
+            uint4_t wv[kU][kMats][kRows];
+            if (kPre != kPreNone && have_pre && c == 0 && unit == unit_first) {
+#pragma unroll
+                for (int u = 0; u < kU; u++)
+#pragma unroll
+                    for (int m = 0; m < kMats; m++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[(u * kMats + m) * kRows + r];
+            } else if (c + kU <= pieces_full) {
+                // full burst: addresses differ by compile-time offsets
+#pragma unroll
+                for (int u = 0; u < kU; u++)
+#pragma unroll
+                    for (int m = 0; m < kMats; m++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++)
+                            wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + (size_t)(c + u) * kPiece + lane * kVec);
+            } else {
+                // tail burst: pieces past the end are skipped, the partial last piece is clamped to valid
+                // weights (they meet zeros of the padded x)
+#pragma unroll
+                for (int u = 0; u < kU; u++) {
+                    const int kk = min((c + u) * kPiece + lane * kVec, K - kVec);
+#pragma unroll
+                    for (int m = 0; m < kMats; m++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++) {
+                            if (c + u < pieces) wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + kk);
+                            else wv[u][m][r] = uint4_t{0u, 0u, 0u, 0u};
+                        }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kU; u++) {
+                if (c + u < pieces) {
+                    float xv[kVec];
+                    load_x<XT, kVec>(xs + (c + u) * kPiece + lane * kVec, xv);
+#pragma unroll
+                    for (int m = 0; m < kMats; m++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++) {
+                            float wf[kVec];
+                            WVec<WT>::unpack(wv[u][m][r], wf);
+#pragma unroll
+                            for (int i = 0; i < kVec; i++) acc[m][r] = fmaf(wf[i], xv[i], acc[m][r]);
+                        }
+                }
+            }
+        }
+
+        // ---- reduce (valid in lane 63) and epilogue ----
+        float v[kMats][kRows];
+#pragma unroll
+        for (int m = 0; m < kMats; m++)
+#pragma unroll
+            for (int r = 0; r < kRows; r++) {
+                v[m][r] = wave_sum_lane63(acc[m][r]);
+                if (p.round_y) v[m][r] = f16r(v[m][r]); // tensor.rs:1623-1643
+            }
+        if (lane == 63) {
+            if constexpr (kEpi == kEpiStore) {
+                act_store1<kDev>(p.y + row0, v[0][0]);
+            } else if constexpr (kEpi == kEpiSilu) {
+                const float g = v[0][0];
+                const float u = v[1][0];
+                const float sg = g / (1.0f + expf(-g)); // tensor.rs:826-827
+                const float mval = sg * u;              // tensor.rs:729
+                act_store1<kDev>(p.y + row0, p.x_f16 ? f16r(mval) : mval); // transformer.rs:563-565 (cast to w2's dtype)
+            } else { // kEpiRopeKv: rows [0, dim) = wq, [dim, 2 dim) = wk, [2 dim, 3 dim) = wv
+                // q and the cache rows are read by the attention kernel, a later launch: ordinary stores
+                const int which = row0 / p.dim;
+                const int jdx = row0 - which * p.dim;
+                const int head = jdx / p.head_dim;
+                const int jj = jdx - head * p.head_dim;
+                float a = v[0][0], b = v[0][kRows - 1];
+                if (which < 2) {
+                    float ra, rb;
+                    rope_pair(a, b, rope_f[jj >> 1], ra, rb);
+                    a = ra;
+                    b = rb;
+                }
+                if (which == 0) {
+                    *reinterpret_cast<float2 *>(p.y + jdx) = make_float2(a, b);
+                } else {
+                    void *cache = which == 1 ? p.cache_k : p.cache_v;
+                    const size_t idx = ((size_t)head * p.max_seq_len + pos) * p.head_dim + jj;
+                    if (p.cache_f16) {
+                        half2_t hv;
+                        hv[0] = (half_t)a; // Tensor::set_f32 on an f16 cache (tensor.rs:373-376)
+                        hv[1] = (half_t)b;
+                        *reinterpret_cast<half2_t *>(reinterpret_cast<half_t *>(cache) + idx) = hv;
+                    } else {
+                        *reinterpret_cast<float2 *>(reinterpret_cast<float *>(cache) + idx) = make_float2(a, b);
+                    }
+                }
+            }
+        }
+    }
+}
+
+} // namespace rlh

@@ -54,6 +54,25 @@ hipError_t launch_gemv(const GemvParams &p, int epilogue, hipStream_t s);
 // bytes of dynamic LDS launch_gemv will request for a given k (for capability checks)
 size_t gemv_lds_bytes(int k, int w_is_f16, int x_f16);
 
+// ---- the matrix-vector phases of one transformer block as one launch (decode_fused.hip) ----
+constexpr int kFusedGroups = 16; // arrival counters of the first barrier level
+// Barrier words in device memory, zero when created: kFusedGroups group counters, the top counter, the generation word and
+// the error word, each on its own 128-byte line.
+struct FusedBarrierState {
+    unsigned words[(kFusedGroups + 3) * 32];
+};
+struct FusedLayerParams {
+    GemvParams wo, w13, w2; // kEpiStore, kEpiSilu, kEpiStore
+    GemvParams last;        // what follows w2: the next block's wq|wk|wv (kEpiRopeKv) or the output head (kEpiStore, fp32 x)
+    int last_kind;          // 0: wq|wk|wv, 1: head with f16 weights, 2: head with f32 weights
+    int n_phases;           // 4, or 3 to stop after w2
+    FusedBarrierState *barrier;
+    long long limit_ticks;  // bound of every barrier wait in 100 MHz wall-clock ticks
+};
+// blocks_out: the grid to launch with (all of it must be resident at once; bounded by the device's capacity)
+hipError_t fused_layer_grid(const FusedLayerParams &p, int compute_units, int *blocks_out);
+hipError_t launch_fused_layer(const FusedLayerParams &p, int blocks, hipStream_t s);
+
 struct AttnDecodeParams {
     const float *q;           // [n_heads x head_dim] f32 (after RoPE)
     const void *cache_k;      // this layer: [n_heads x max_seq_len x head_dim]
