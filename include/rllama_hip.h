@@ -258,6 +258,17 @@ int  rlh_rope_kvwrite(rlh_tensor *q, const rlh_tensor *k, const rlh_tensor *v, r
  * finite where the reference overflows to NaN (scores above ln(FLT_MAX)). */
 int  rlh_attn_decode(rlh_tensor *out, const rlh_tensor *q, const rlh_tensor *cache_k, const rlh_tensor *cache_v, int n_heads, int max_seq_len,
                      int T, int n_splits, int round_out);
+/* rlh_attn_decode for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and bit-identical
+ * results, but the work memory (arrival counters, the position word and the partial triples of a split sequence) is a
+ * static device array of 4 MiB + 4.25 KiB inside the library, which every GPU the library runs on holds until the process
+ * ends; rlh_init looks its address up once per device.  Nothing is allocated or freed by the call (no hipMalloc, no
+ * hipFree, no memset node: the counters are cleared by a small fill kernel).  Limits: n_heads * n_splits * (head_dim + 2)
+ * <= 1,048,576 floats (e.g. 64 heads of 128 dims with 64 splits need 532,480), else RLH_ERR_UNSUPPORTED.  All calls on one
+ * GPU share the array, which keeps the last call's contents: calls that overlap on one GPU (two contexts on the same
+ * device, or a captured graph replayed while another call runs) race. */
+int  rlh_attn_decode_noalloc(rlh_tensor *out, const rlh_tensor *q, const rlh_tensor *cache_k, const rlh_tensor *cache_v, int n_heads,
+                             int max_seq_len, int T, int n_splits, int round_out);
 /* The attention block of a multi-token forward at start_pos 0 between the projections and wo (src/transformer.rs:704-796):
  * RoPE on the q and k columns of qkv, k and v into the cache planes at positions 0..n-1, causal attention per head, heads
  * concatenated and rounded to f16.  qkv: f16 [n x 3 dim] (columns [0, dim) wq's output, [dim, 2 dim) wk's, [2 dim, 3 dim)

@@ -393,6 +393,11 @@ class Tensor:
         check(self._lib.rlh_attn_decode(out._h, self._h, cache_k._h, cache_v._h, n_heads, max_seq_len, T, n_splits, 1 if round_out else 0))
         return out
 
+    def attn_decode_noalloc(self, out: "Tensor", cache_k: "Tensor", cache_v: "Tensor", n_heads: int, max_seq_len: int, T: int,
+                            n_splits: int = 0, round_out: bool = False) -> None:
+        """attn_decode into a tensor the caller made, on the library's static work memory: the call allocates nothing."""
+        check(self._lib.rlh_attn_decode_noalloc(out._h, self._h, cache_k._h, cache_v._h, n_heads, max_seq_len, T, n_splits, 1 if round_out else 0))
+
     def attn_prefill(self, cache_k: "Tensor", cache_v: "Tensor", n_heads: int, max_seq_len: int) -> "Tensor":
         """self = qkv f16 [n x 3 dim]: RoPE, cache write and causal attention of a prompt (src/transformer.rs:704-796) -> f16 [n x dim]."""
         out = Tensor.zeros(self.ctx, self._rows, self._cols // 3, TensorDType.Float16)

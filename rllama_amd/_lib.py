@@ -90,6 +90,7 @@ SIGNATURES = {
     "rlh_silu_mul": (C.c_int, [_vp, _vp, _vp]),
     "rlh_rope_kvwrite": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int]),
     "rlh_attn_decode": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "rlh_attn_decode_noalloc": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "rlh_attn_prefill": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, C.c_int]),
     "rlh_argmax_greedy": (C.c_int, [_vp, C.c_float, _i32p]),
     "rlh_model_time_kernel": (C.c_int, [_vp, _vp, C.c_int, C.c_int, C.c_int, _fp, C.POINTER(C.c_uint64)]),

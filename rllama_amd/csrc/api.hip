@@ -176,6 +176,11 @@ extern "C" int rlh_init(int device_ordinal, int verbose, rlh_ctx **out) {
         delete c;
         return fail(RLH_ERR_HIP, "rlh_init: hipStreamCreate: %s", hipGetErrorString(e));
     }
+    if (int rc = noalloc_setup(c); rc != RLH_OK) {
+        (void)hipStreamDestroy(c->stream);
+        delete c;
+        return rc;
+    }
     if (verbose) {
         fprintf(stderr, "rllama_hip: device %d %s (%s), %d CUs, %.1f GB HBM\n", device_ordinal, c->prop.name, c->prop.gcnArchName,
                 c->prop.multiProcessorCount, (double)c->prop.totalGlobalMem / 1e9);

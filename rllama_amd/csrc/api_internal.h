@@ -42,6 +42,7 @@ struct rlh_ctx {
     hipDeviceProp_t prop;
     std::recursive_mutex mu;
     OpScratch ops;
+    void *noalloc_scratch = nullptr; // this device's address of the library's static work memory (api_ops.hip)
 };
 
 struct rlh_tensor {
@@ -64,6 +65,9 @@ struct CtxLock {
 
 namespace rlh {
 void ops_release(rlh_ctx *ctx); // frees the op-level work memory (rlh_shutdown)
+// looks up the context's device address of the static work memory of rlh_attn_decode_noalloc; rlh_init calls it with the
+// device current
+int noalloc_setup(rlh_ctx *ctx);
 // how many blocks per head the decode attention uses at sequence length T
 int attn_splits_rule(int T, int single_max, int chunk, int max_splits);
 } // namespace rlh

@@ -511,3 +511,50 @@ extern "C" int rlh_argmax_greedy(const rlh_tensor *logits, float temperature, in
     HIP_TRY(hipStreamSynchronize(st));
     return RLH_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// rlh_attn_decode without any allocation: the work memory is a static device array
+// ------------------------------------------------------------------------------------------------
+// Layout of the array: arrival counters [kOpMaxHeads], the position word block, then the partial triples.
+constexpr size_t kStaticTicketsBytes = sizeof(unsigned) * kOpMaxHeads;
+constexpr size_t kStaticStateOffset = kStaticTicketsBytes;
+constexpr size_t kStaticWsOffset = kStaticStateOffset + 256;
+constexpr size_t kStaticWsFloats = (size_t)1 << 20; // 4 MiB of partial triples: n_heads * n_splits * (head_dim + 2) floats at most
+constexpr size_t kStaticScratchBytes = kStaticWsOffset + kStaticWsFloats * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace rlh {
+// The array's name is only a host-side stand-in; every device holds its own copy at its own address.  This looks the
+// address up for the context's device (current when rlh_init calls this) and keeps it in the context.
+int noalloc_setup(rlh_ctx *ctx) {
+    void *ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+        return fail(RLH_ERR_HIP, "rlh_init: hipGetSymbolAddress(scratch) on device %d: %s", ctx->device, hipGetErrorString(e));
+    }
+    ctx->noalloc_scratch = ptr;
+    return RLH_OK;
+}
+} // namespace rlh
+
+extern "C" int rlh_attn_decode_noalloc(rlh_tensor *out, const rlh_tensor *q, const rlh_tensor *cache_k, const rlh_tensor *cache_v, int n_heads,
+                                       int max_seq_len, int T, int n_splits, int round_out) {
+    int hd = 0;
+    int rc = check_attn_decode("rlh_attn_decode_noalloc", out, q, cache_k, cache_v, n_heads, max_seq_len, T, &n_splits, &hd);
+    if (rc != RLH_OK) return rc;
+    const size_t need = attn_decode_workspace_floats(n_heads, hd, n_splits);
+    if (need > kStaticWsFloats) {
+        return fail(RLH_ERR_UNSUPPORTED,
+                    "rlh_attn_decode_noalloc: %d heads x %d splits x (%d + 2) floats = %zu exceed the static work memory of %zu floats; use fewer "
+                    "splits or rlh_attn_decode",
+                    n_heads, n_splits, hd, need, kStaticWsFloats);
+    }
+    rlh_ctx *ctx = out->ctx;
+    CtxLock lock(ctx);
+    unsigned char *base = static_cast<unsigned char *>(ctx->noalloc_scratch); // this device's address of `scratch`, from rlh_init
+    if (!base) return fail(RLH_ERR_STATE, "rlh_attn_decode_noalloc: the context holds no address of the static work memory");
+    HIP_TRY(enqueue_attn_decode(ctx, out, q, cache_k, cache_v, n_heads, hd, max_seq_len, T, n_splits, round_out,
+                                reinterpret_cast<DecodeState *>(base + kStaticStateOffset), reinterpret_cast<float *>(base + kStaticWsOffset),
+                                reinterpret_cast<unsigned *>(base)));
+    return RLH_OK;
+}

@@ -129,6 +129,7 @@ extern "C" {
     pub fn rlh_silu_mul(dst: *mut rlh_tensor, gate: *const rlh_tensor, up: *const rlh_tensor) -> c_int;
     pub fn rlh_rope_kvwrite(q: *mut rlh_tensor, k: *const rlh_tensor, v: *const rlh_tensor, cache_k: *mut rlh_tensor, cache_v: *mut rlh_tensor, n_heads: c_int, max_seq_len: c_int, pos: c_int) -> c_int;
     pub fn rlh_attn_decode(out: *mut rlh_tensor, q: *const rlh_tensor, cache_k: *const rlh_tensor, cache_v: *const rlh_tensor, n_heads: c_int, max_seq_len: c_int, T: c_int, n_splits: c_int, round_out: c_int) -> c_int;
+    pub fn rlh_attn_decode_noalloc(out: *mut rlh_tensor, q: *const rlh_tensor, cache_k: *const rlh_tensor, cache_v: *const rlh_tensor, n_heads: c_int, max_seq_len: c_int, T: c_int, n_splits: c_int, round_out: c_int) -> c_int;
     pub fn rlh_attn_prefill(out: *mut rlh_tensor, qkv: *const rlh_tensor, cache_k: *mut rlh_tensor, cache_v: *mut rlh_tensor, n_heads: c_int, max_seq_len: c_int) -> c_int;
     pub fn rlh_argmax_greedy(logits: *const rlh_tensor, temperature: c_float, token: *mut i32) -> c_int;
     pub fn rlh_model_time_kernel(model: *mut rlh_model, caches: *mut rlh_caches, which: c_int, T: c_int, iters: c_int, us_per_launch: *mut c_float, bytes_per_launch: *mut u64) -> c_int;
