@@ -250,6 +250,9 @@ def main() -> int:
                 continue
             us, nbytes = model.time_kernel(which, T_mid, args.kernel_iters, caches)
             out["kernels"][name] = {"us": round(us, 2), "bytes": nbytes}
+        if not args.kernel or args.kernel == "fused_layer":
+            us, nbytes = model.time_kernel(ra.Transformer.FUSED_LAYER_KERNEL, T_mid, args.kernel_iters, caches)
+            out["kernels"]["fused_layer"] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
         print(json.dumps(out))
         return 0
 

@@ -287,7 +287,8 @@ int  rlh_argmax_greedy(const rlh_tensor *logits, float temperature, int32_t *tok
  * ---------------------------------------------------------------------------------------------- */
 /* One kernel of the token step, cycling through the layers so that every launch streams different weights.
  * which: 0 = attention_norm + wq|wk|wv + RoPE + cache write, 1 = single-query attention at sequence length T,
- * 2 = wo + residual, 3 = ffn_norm + w1|w3 + SiLU*gate, 4 = w2 + residual, 5 = final norm + output head.
+ * 2 = wo + residual, 3 = ffn_norm + w1|w3 + SiLU*gate, 4 = w2 + residual, 5 = final norm + output head,
+ * 6 = the fused layer kernel (2, 3, 4 and the next layer's 0 as one launch).
  * bytes_per_launch (may be NULL): the algorithmic bytes of one launch (weights once + vectors).
  * The launches use the model's token-step state and activation buffers as they are and leave them overwritten (position
  * T - 1, a fixed token id), and which = 0 writes the K / V rows of position T - 1 of every layer of `caches`: use caches

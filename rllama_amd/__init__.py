@@ -256,6 +256,7 @@ class Transformer:
         return out, ms.value
 
     STEP_KERNELS = ("qkv_rope_kvwrite", "attn_decode", "wo_residual", "w13_silu", "w2_residual", "head")
+    FUSED_LAYER_KERNEL = 6   # wo + w1|w3 + w2 + the next layer's wq|wk|wv as one launch
 
     def time_kernel(self, which: int, T: int, iters: int, caches: TransformerCaches):
         """(microseconds per launch, algorithmic bytes per launch) of one token-step kernel, HIP-event timed."""

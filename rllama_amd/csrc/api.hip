@@ -109,8 +109,9 @@ struct rlh_model {
     bool capturing = false;    // a decode step is being recorded into a HIP graph
     // fused layer kernel (decode_fused.hip), RLLAMA_HIP_FUSED=1; otherwise one launch per matrix-vector product
     bool fused_layers = getenv("RLLAMA_HIP_FUSED") && atoi(getenv("RLLAMA_HIP_FUSED")) != 0;
-    FusedBarrierState *fused_barrier = nullptr;
-    long long fused_limit_ticks = 20000000; // 200 ms at the 100 MHz wall clock
+    FusedBarrierState *fused_barrier = nullptr; // one per kernel variant: a barrier's counters assume one grid size for its lifetime
+    // bound of every barrier wait: 200 ms at the 100 MHz wall clock (RLLAMA_HIP_FUSED_LIMIT_TICKS overrides it; tests use 0)
+    long long fused_limit_ticks = getenv("RLLAMA_HIP_FUSED_LIMIT_TICKS") ? atoll(getenv("RLLAMA_HIP_FUSED_LIMIT_TICKS")) : 20000000;
     int fused_blocks[4] = {0, 0, 0, 0};     // grid per kernel variant (last phase wq|wk|wv / f16 head / f32 head / none), 0 = not yet asked
     bool fused_used = false;                // a fused kernel was enqueued since the error word was last checked
     bool attn_lds_stage = getenv("RLLAMA_HIP_ATTN_LDS") && atoi(getenv("RLLAMA_HIP_ATTN_LDS")) != 0; // comparison variant of the decode attention
@@ -341,7 +342,7 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     B((void **)&m->prompt_dev, sizeof(int32_t) * m->prompt_cap);
     B((void **)&m->attn_ws, sizeof(float) * attn_decode_workspace_floats(prm->n_heads, hd, m->max_splits));
     B((void **)&m->attn_tickets, sizeof(unsigned) * (size_t)prm->n_heads);
-    B((void **)&m->fused_barrier, sizeof(FusedBarrierState));
+    B((void **)&m->fused_barrier, sizeof(FusedBarrierState) * 4);
     if (rc == RLH_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(RLH_ERR_HIP, "rlh_model_create: hipDeviceSynchronize failed");
     if (rc != RLH_OK) {
         rlh_model_free(m);
@@ -822,9 +823,10 @@ static int enqueue_fused_layer(rlh_model *m, rlh_caches *c, int l, bool with_hea
         F.n_phases = 3;
         F.last_kind = 0;
     }
-    F.barrier = m->fused_barrier;
+    const int variant = F.n_phases == 3 ? 3 : F.last_kind;
+    F.barrier = m->fused_barrier + variant;
     F.limit_ticks = m->fused_limit_ticks;
-    int &blocks = m->fused_blocks[F.n_phases == 3 ? 3 : F.last_kind];
+    int &blocks = m->fused_blocks[variant];
     if (blocks == 0) HIP_TRY(fused_layer_grid(F, m->ctx->prop.multiProcessorCount, &blocks));
     HIP_TRY(launch_fused_layer(F, blocks, m->ctx->stream));
     m->fused_used = true;
@@ -836,11 +838,12 @@ static int enqueue_fused_layer(rlh_model *m, rlh_caches *c, int l, bool with_hea
 static int check_fused_barrier(rlh_model *m) {
     if (!m->fused_used) return RLH_OK;
     m->fused_used = false;
+    FusedBarrierState host[4];
+    HIP_TRY(hipMemcpy(host, m->fused_barrier, sizeof(host), hipMemcpyDeviceToHost));
     unsigned err = 0;
-    const size_t err_off = sizeof(unsigned) * (size_t)(kFusedGroups + 2) * 32;
-    HIP_TRY(hipMemcpy(&err, (const char *)m->fused_barrier + err_off, sizeof(err), hipMemcpyDeviceToHost));
+    for (const FusedBarrierState &b : host) err |= b.words[(kFusedGroups + 2) * 32];
     if (err == 0) return RLH_OK;
-    HIP_TRY(hipMemset(m->fused_barrier, 0, sizeof(FusedBarrierState)));
+    HIP_TRY(hipMemset(m->fused_barrier, 0, sizeof(host)));
     m->next_pos = -1;
     m->greedy_caches = nullptr;
     return fail(RLH_ERR_HIP, "a device-wide barrier of the fused layer kernel did not complete within its time limit (not every workgroup "
@@ -1253,7 +1256,7 @@ extern "C" int rlh_forward(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     if (rc != RLH_OK) return rc;
     HIP_TRY(hipMemcpyAsync(logits_out, m->logits, sizeof(float) * (size_t)m->prm.vocab_size, hipMemcpyDeviceToHost, m->ctx->stream));
     HIP_TRY(hipStreamSynchronize(m->ctx->stream));
-    return RLH_OK;
+    return check_fused_barrier(m);
 }
 
 // forward + the device pick at top_k = 1 on logits * scale
@@ -1270,7 +1273,7 @@ static int forward_greedy_scaled(rlh_model *m, rlh_caches *c, const int32_t *tok
     HIP_TRY(hipStreamSynchronize(st));
     m->next_pos = start_pos + n;
     m->greedy_caches = c;
-    return RLH_OK;
+    return check_fused_barrier(m);
 }
 
 extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, int32_t *next_token) {
@@ -1431,7 +1434,7 @@ extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *p
     HIP_TRY(e);
     m->next_pos = n_prompt + n_new - 1;
     m->greedy_caches = c;
-    return RLH_OK;
+    return check_fused_barrier(m);
 }
 
 extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32_t *out_tokens, float *ms_total) {
@@ -1469,7 +1472,7 @@ extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32
     HIP_TRY(e2);
     if (ms_total) *ms_total = ms;
     m->next_pos += n_steps;
-    return RLH_OK;
+    return check_fused_barrier(m);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1479,7 +1482,9 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
     if (!m || !c || !us_per_launch || iters < 1) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad argument");
     if (c->model != m || c->model_uid != m->uid) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: caches belong to another model");
     if (!model_ready(m)) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: model has tensors that were never set");
-    if (T < 1 || T > m->prm.max_seq_len || which < kStepQkv || which > kStepHead) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad T or kernel id");
+    constexpr int kStepFused = 6; // wo + w1|w3 + w2 + the next layer's wq|wk|wv as one launch
+    if (T < 1 || T > m->prm.max_seq_len || which < kStepQkv || which > kStepFused) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad T or kernel id");
+    if (which == kStepFused && m->prm.n_layers < 2) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: the fused layer kernel needs two layers");
     CtxLock lock(m->ctx);
     hipStream_t st = m->ctx->stream;
     const uint64_t d = (uint64_t)m->prm.dim, F = (uint64_t)m->prm.ffn_hidden, V = (uint64_t)m->prm.vocab_size;
@@ -1492,6 +1497,7 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
         case kStepWo: *bytes_per_launch = d * d * es + d * 4 + 2 * d * 4; break;
         case kStepW13: *bytes_per_launch = 2 * F * d * es + d * 4 + d * 4 + F * 4; break;
         case kStepW2: *bytes_per_launch = d * F * es + F * 4 + 2 * d * 4; break;
+        case kStepFused: *bytes_per_launch = (4 * d * d + 3 * d * F) * es + 8 * d * 4 + 2 * F * 4 + 2 * d * es; break;
         default: *bytes_per_launch = V * d * (m->output.f16 ? 2 : 4) + d * 4 + d * 4 + V * 4; break;
         }
     }
@@ -1504,9 +1510,11 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
     HIP_TRY(hipEventCreate(&e1));
     int rc = RLH_OK;
     const int L = m->prm.n_layers;
-    for (int i = 0; rc == RLH_OK && i < (L < 4 ? L : 4); i++) rc = enqueue_step_kernel(m, c, i % L, which, T); // warm-up
+    // (the fused kernel cycles over layers 0 .. L - 2, whose last phase is the next layer's wq|wk|wv)
+    auto one = [&](int i) { return which == kStepFused ? enqueue_fused_layer(m, c, i % (L - 1), true) : enqueue_step_kernel(m, c, i % L, which, T); };
+    for (int i = 0; rc == RLH_OK && i < (L < 4 ? L : 4); i++) rc = one(i); // warm-up
     hipError_t e = hipEventRecord(e0, st);
-    for (int i = 0; rc == RLH_OK && e == hipSuccess && i < iters; i++) rc = enqueue_step_kernel(m, c, i % L, which, T);
+    for (int i = 0; rc == RLH_OK && e == hipSuccess && i < iters; i++) rc = one(i);
     if (e == hipSuccess) e = hipEventRecord(e1, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     float ms = 0.0f;
@@ -1516,7 +1524,7 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
     if (rc != RLH_OK) return rc;
     HIP_TRY(e);
     *us_per_launch = ms * 1000.0f / (float)iters;
-    return RLH_OK;
+    return check_fused_barrier(m);
 }
 
 extern "C" int rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int round_x, int round_y, int n_buffers, int iters, float *us_per_launch) {

@@ -3,15 +3,22 @@
 // A token step is a chain of dependent matrix-vector products (Noeda/rllama, transformer.rs:424-446, 536-583, 657-820):
 // wo -> (residual, ffn_norm) w1|w3 -> w2 -> (residual, attention_norm of the next block) wq|wk|wv, or the output head after
 // the last block.  As separate launches every link costs the fixed price of a kernel boundary (about 3 us during which no
-// weight byte moves), four times per block.  Here the four products are phases of one kernel on one resident grid:
+// weight byte moves).  Here the four products are phases of one kernel on one resident grid:
 //   * between two phases all workgroups meet at a device-wide barrier (two levels of arrival counters, so that no counter
-//     sees more than a few dozen atomics; about 2 us from the last arrival to the last release);
-//   * the weights of a phase do not depend on the activations, so every wavefront requests the first burst of its first
-//     row of the NEXT phase before it waits at the barrier: the memory system keeps streaming while the hand-over of the
-//     activation vector (a few KB) takes place;
+//     sees more than a few dozen atomics);
+//   * the weights of a phase do not depend on the activations, so every wavefront requests the first burst(s) of its first
+//     row(s) of the NEXT phase before it waits at the barrier;
 //   * activation vectors that cross the barrier are written and read at device scope (gemv_device.h), everything else --
 //     the weight stream, q and the cache rows for the attention kernel that follows -- as in the stand-alone kernels.
 // The arithmetic of every phase is gemv_body, the same code the stand-alone kernels run: results are bit-identical.
+//
+// MEASURED, AND NOT THE DEFAULT: on the 7B shape the fused launch takes 82 us against 76 us for the four kernels it
+// replaces.  Per-workgroup time stamps show why: the phases themselves run at the streaming rate, but the workgroups of a
+// phase finish up to 9 us apart (the memory system does not serve them evenly), the barrier completes 1.5 - 4 us after the
+// LAST arrival, and what a wavefront requested ahead when IT arrived has long landed by then -- one, two, three or four
+// bursts ahead make no difference -- so the memory system idles about as long as across a kernel boundary, and the
+// device-scope hand-over of the activation vector costs more than the L2-cached reads of a fresh kernel.  It is kept behind
+// RLLAMA_HIP_FUSED=1 as the reference point for that measurement.
 //
 // Every wait is bounded by the wall clock: a barrier that does not complete within the limit (a workgroup that never became
 // resident) raises the error word, every workgroup leaves, and the host reports the failure.
@@ -22,6 +29,10 @@
 namespace rlh {
 
 constexpr int kFusedLine = 32;  // counters sit on separate 128-byte lines
+#ifndef RLH_FUSED_PREFETCH
+#define RLH_FUSED_PREFETCH 1
+#endif
+constexpr int kFusedPrefetch = RLH_FUSED_PREFETCH; // bursts of the next phase every wavefront requests before it waits at a barrier
 
 __device__ __forceinline__ unsigned bar_load(const unsigned *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void bar_store(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -84,8 +95,8 @@ __global__ __launch_bounds__(kGemvThreads) void fused_layer_kernel(FusedLayerPar
         s_abort = 0;
         bar.init(P.barrier, P.limit_ticks);
     }
-    uint4_t wpre[kGemvBurst];
-    bool have = gemv_issue_first_burst<WT, kEpiStore, true>(P.wo, wpre);
+    uint4_t wpre[kFusedPrefetch][kGemvBurst];
+    unsigned have = gemv_issue_bursts<WT, kEpiStore, true, kFusedPrefetch>(P.wo, wpre);
     __syncthreads();
 
     // End of a phase: this wavefront's activation stores are acknowledged, the workgroup arrives, the next phase's first
@@ -101,23 +112,23 @@ __global__ __launch_bounds__(kGemvThreads) void fused_layer_kernel(FusedLayerPar
     };
 
     // wo (transformer.rs:783-819)
-    gemv_body<WT, XT, kEpiStore, true, true, kPreGiven>(P.wo, smem_raw, red, rope_f, wpre, have);
-    if (!hand_over([&]() { return gemv_issue_first_burst<WT, kEpiSilu, true>(P.w13, wpre); })) return;
+    gemv_body<WT, XT, kEpiStore, true, true, kPreGiven, true, kFusedPrefetch>(P.wo, smem_raw, red, rope_f, wpre, have);
+    if (!hand_over([&]() { return gemv_issue_bursts<WT, kEpiSilu, true, kFusedPrefetch>(P.w13, wpre); })) return;
     // h = x + wo(att), ffn_norm, w1|w3, SiLU * gate (transformer.rs:442-443, 537-565)
-    gemv_body<WT, XT, kEpiSilu, true, true, kPreGiven>(P.w13, smem_raw, red, rope_f, wpre, have);
-    if (!hand_over([&]() { return gemv_issue_first_burst<WT, kEpiStore, true>(P.w2, wpre); })) return;
+    gemv_body<WT, XT, kEpiSilu, true, true, kPreGiven, true, kFusedPrefetch>(P.w13, smem_raw, red, rope_f, wpre, have);
+    if (!hand_over([&]() { return gemv_issue_bursts<WT, kEpiStore, true, kFusedPrefetch>(P.w2, wpre); })) return;
     // w2 (transformer.rs:568-570)
-    gemv_body<WT, XT, kEpiStore, true, true, kPreGiven>(P.w2, smem_raw, red, rope_f, wpre, have);
+    gemv_body<WT, XT, kEpiStore, true, true, kPreGiven, true, kFusedPrefetch>(P.w2, smem_raw, red, rope_f, wpre, have);
     if (P.n_phases < 4) return;
     if constexpr (kLast == 0) {
-        if (!hand_over([&]() { return gemv_issue_first_burst<WT, kEpiRopeKv, true>(P.last, wpre); })) return;
+        if (!hand_over([&]() { return gemv_issue_bursts<WT, kEpiRopeKv, true, kFusedPrefetch>(P.last, wpre); })) return;
         // x = h + w2(...), the next block's attention_norm, wq|wk|wv, RoPE, cache write (transformer.rs:445, 432, 665-761)
-        gemv_body<WT, XT, kEpiRopeKv, true, true, kPreGiven>(P.last, smem_raw, red, rope_f, wpre, have);
+        gemv_body<WT, XT, kEpiRopeKv, true, true, kPreGiven, true, kFusedPrefetch>(P.last, smem_raw, red, rope_f, wpre, have);
     } else {
         using HT = typename std::conditional<kLast == 1, half_t, float>::type;
-        if (!hand_over([&]() { return gemv_issue_first_burst<HT, kEpiStore, true>(P.last, wpre); })) return;
+        if (!hand_over([&]() { return gemv_issue_bursts<HT, kEpiStore, true, kFusedPrefetch>(P.last, wpre); })) return;
         // x = h + w2(...), final norm, output head on fp32 activations (transformer.rs:445, 378-381)
-        gemv_body<HT, float, kEpiStore, true, true, kPreGiven>(P.last, smem_raw, red, rope_f, wpre, have);
+        gemv_body<HT, float, kEpiStore, true, true, kPreGiven, true, kFusedPrefetch>(P.last, smem_raw, red, rope_f, wpre, have);
     }
 }
 

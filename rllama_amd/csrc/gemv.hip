@@ -35,8 +35,8 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     // (measured: issuing the first burst behind the prologue's loads is worth 1 % on the w1|w3 product, nothing or a loss on
     // the others, so only that instantiation does it)
     constexpr int kPre = (RLH_GEMV_PRELOAD && kEpi == kEpiSilu) ? kPreSelf : kPreNone;
-    uint4_t wpre[kGemvBurst];
-    gemv_body<WT, XT, kEpi, kStream, false, kPre>(p, smem_raw, red, rope_f, wpre, false);
+    uint4_t wpre[1][kGemvBurst];
+    gemv_body<WT, XT, kEpi, kStream, false, kPre>(p, smem_raw, red, rope_f, wpre, 0u);
 }
 
 template <typename WT, typename XT, int kEpi>

@@ -5,7 +5,21 @@
 #include "kernels.h"
 #include "device_utils.h"
 
+#include <type_traits>
+#include <utility>
+
 namespace rlh {
+
+// f(integral_constant<int, 0>), f(integral_constant<int, 1>), ...: a loop whose index is a compile-time constant in every
+// iteration (register arrays indexed by it stay in registers)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int kN, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, kN>{});
+}
 
 // Launch shape (overridable at compile time for tuning runs).
 #ifndef RLH_GEMV_WAVES
@@ -90,23 +104,24 @@ __device__ __forceinline__ float wave_sum_lane63(float v) {
 // ---- activations that cross workgroups inside one launch --------------------------------------------------------------
 // Between kernels the launch boundary makes every store visible.  Inside the fused layer kernel an activation vector is
 // written by some workgroups and read by all of them after a device-wide barrier, and the eight L2 caches of the part are
-// not coherent with each other for ordinary accesses: such vectors are therefore stored and loaded at device scope
-// (write-through stores, loads that do not take a stale L2 line).  kDev selects that form.
+// not coherent with each other for ordinary accesses: such vectors are stored (kDev) and loaded (kDevLoad) at device scope
+// -- write-through stores that are in memory once acknowledged, loads that do not take a stale L2 line.  Measured
+// alternatives for the reading side: an acquire fence at device scope followed by ordinary loads costs 9 us per barrier
+// (it invalidates the L2 under the weight stream); four-byte device-scope loads cost 3 us per phase (512 workgroups
+// fetching the same few KB dword by dword from memory); 16-byte ones about 1 us.
+// Device-scope 16-byte loads are written as inline assembly (the compiler offers device scope only for scalar types): a
+// batch is issued with act_issue4, then act_wait8 waits for everything outstanding and ties the destination registers to the
+// wait, so that no use of them can be scheduled in front of it.  The ordinary form is a plain load and no wait.
 template <bool kDev>
-__device__ __forceinline__ float4_t act_load4(const float4_t *p) {
-    if constexpr (kDev) {
-        const unsigned long long *q = reinterpret_cast<const unsigned long long *>(p);
-        const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        float4_t v;
-        v[0] = __builtin_bit_cast(float, (unsigned)(lo & 0xffffffffull));
-        v[1] = __builtin_bit_cast(float, (unsigned)(lo >> 32));
-        v[2] = __builtin_bit_cast(float, (unsigned)(hi & 0xffffffffull));
-        v[3] = __builtin_bit_cast(float, (unsigned)(hi >> 32));
-        return v;
-    } else {
-        return *p;
-    }
+__device__ __forceinline__ void act_issue4(float4_t &dst, const float4_t *p) {
+    if constexpr (kDev) asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(dst) : "v"(p) : "memory");
+    else dst = *p;
+}
+template <bool kDev, int kN>
+__device__ __forceinline__ void act_wait(float4_t (&v)[kN]) {
+    static_assert(kN == 8, "batches of eight");
+    if constexpr (kDev)
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])::"memory");
 }
 template <bool kDev>
 __device__ __forceinline__ float act_load1(const float *p) {
@@ -116,11 +131,11 @@ __device__ __forceinline__ float act_load1(const float *p) {
 template <bool kDev>
 __device__ __forceinline__ void act_store4(float4_t *p, float4_t v) {
     if constexpr (kDev) {
-        unsigned long long *q = reinterpret_cast<unsigned long long *>(p);
-        const unsigned long long lo = (unsigned long long)__builtin_bit_cast(unsigned, v[0]) | ((unsigned long long)__builtin_bit_cast(unsigned, v[1]) << 32);
-        const unsigned long long hi = (unsigned long long)__builtin_bit_cast(unsigned, v[2]) | ((unsigned long long)__builtin_bit_cast(unsigned, v[3]) << 32);
-        __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(q + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float *q = reinterpret_cast<float *>(p);
+        __hip_atomic_store(q, v[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(q + 1, v[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(q + 2, v[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(q + 3, v[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
         *p = v;
     }
@@ -148,35 +163,51 @@ struct GemvShape {
     static constexpr int kPiece = kWave * kVec;                  // elements one wave-wide load covers
 };
 
-// Issues the first burst of this wavefront's first row unit into wpre (kGemvBurst 16-byte loads) if that unit exists and
-// starts with a full burst; returns whether it did.  The loads do not depend on x.
-template <typename WT, int kEpi, bool kStream>
-__device__ __forceinline__ bool gemv_issue_first_burst(const GemvParams &p, uint4_t (&wpre)[kGemvBurst]) {
+// The bursts of a wavefront in the order its main loop takes them: row units unit_first, unit_first + W, ..., and within a
+// unit the pieces 0, kU, 2 kU, ...  This issues the loads of the first kD of them into wpre and returns a mask of those it
+// issued (bit d: burst d is in wpre[d]); a burst that does not exist or is not a full one (the ragged end of a row) is left
+// to the main loop.  The loads do not depend on x.
+template <typename WT, int kEpi, bool kStream, int kD>
+__device__ __forceinline__ unsigned gemv_issue_bursts(const GemvParams &p, uint4_t (&wpre)[kD][kGemvBurst]) {
     using S = GemvShape<WT, kEpi>;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int K = p.k;
-    const int unit_first = blockIdx.x * kGemvWaves + wave;
-    const bool have = unit_first < p.n_rows / S::kRows && S::kU <= K / S::kPiece;
-    if (have) {
-        const WT *wmat[2] = {reinterpret_cast<const WT *>(p.w), reinterpret_cast<const WT *>(p.w_b)};
+    const int pieces = gemv_iters(K, S::kVec);
+    const int pieces_full = K / S::kPiece;
+    const int n_units = p.n_rows / S::kRows;
+    const int W = gridDim.x * kGemvWaves;
+    const WT *wmat[2] = {reinterpret_cast<const WT *>(p.w), reinterpret_cast<const WT *>(p.w_b)};
+    int unit = blockIdx.x * kGemvWaves + wave, c = 0;
+    unsigned mask = 0;
+    static_for<kD>([&](auto dc) {
+        constexpr int d = decltype(dc)::value;
+        if (unit < n_units && c + S::kU <= pieces_full) {
+            mask |= 1u << d;
 #pragma unroll
-        for (int u = 0; u < S::kU; u++)
+            for (int u = 0; u < S::kU; u++)
 #pragma unroll
-            for (int m = 0; m < S::kMats; m++)
+                for (int m = 0; m < S::kMats; m++)
 #pragma unroll
-                for (int r = 0; r < S::kRows; r++)
-                    wpre[(u * S::kMats + m) * S::kRows + r] =
-                        load16<kStream>(wmat[m] + (size_t)(unit_first * S::kRows + r) * K + (size_t)u * S::kPiece + lane * S::kVec);
-    }
-    return have;
+                    for (int r = 0; r < S::kRows; r++)
+                        wpre[d][(u * S::kMats + m) * S::kRows + r] =
+                            load16<kStream>(wmat[m] + (size_t)(unit * S::kRows + r) * K + (size_t)(c + u) * S::kPiece + lane * S::kVec);
+        }
+        c += S::kU;
+        if (c >= pieces) {
+            c = 0;
+            unit += W;
+        }
+    });
+    return mask;
 }
 
 // One GEMV over the whole grid: prologue (x staged in LDS), main loop, epilogue.  `smem_raw` is the block's dynamic LDS
 // (gemv_lds_bytes); `red` 16 floats and `rope_f` 64 float2 of static LDS.  kDev: x / x_add are read and y / x_out written at
-// device scope (see above).  With kPre == kPreGiven, wpre holds the first burst and have_pre says whether it was issued.
-template <typename WT, typename XT, int kEpi, bool kStream, bool kDev, int kPre>
-__device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f, uint4_t (&wpre)[kGemvBurst], bool have_pre) {
+// device scope (see above).  With kPre == kPreGiven, wpre holds the first kD bursts the caller issued and pre_mask says which.
+template <typename WT, typename XT, int kEpi, bool kStream, bool kDev, int kPre, bool kDevLoad = false, int kD = 1>
+__device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f, uint4_t (&wpre)[kD][kGemvBurst],
+                                          unsigned pre_mask) {
     using S = GemvShape<WT, kEpi>;
     constexpr int kVec = S::kVec, kMats = S::kMats, kRows = S::kRows, kU = S::kU, kPiece = S::kPiece;
     XT *xs = reinterpret_cast<XT *>(smem_raw);
@@ -194,10 +225,10 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     if constexpr (kMats == 2) wmat[1] = reinterpret_cast<const WT *>(p.w_b);
     const int unit_first = blockIdx.x * kGemvWaves + wave;
     auto preload = [&]() {
-        if constexpr (kPre == kPreSelf) have_pre = gemv_issue_first_burst<WT, kEpi, kStream>(p, wpre);
+        if constexpr (kPre == kPreSelf) pre_mask = gemv_issue_bursts<WT, kEpi, kStream, kD>(p, wpre);
         __builtin_amdgcn_sched_barrier(0);
     };
-    if constexpr (kPre == kPreNone) have_pre = false;
+    if constexpr (kPre == kPreNone) pre_mask = 0;
 
     // ---- prologue: x = (x_in [+ x_add]) [RMSNorm] [-> f16], staged in LDS, zero padded to kpad ----
     // All global loads of a batch are issued before any is consumed (one exposed memory latency per batch).
@@ -210,15 +241,22 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     if (p.norm_w != nullptr && n4 <= kGemvPrologueVecs * kGemvThreads) {
         // RMSNorm::forward (transformer.rs:476-480): (x * rsqrt(mean(x^2) + eps)) * w, x kept in registers
         const float4_t *w4 = reinterpret_cast<const float4_t *>(p.norm_w);
-        float4_t xv[kGemvPrologueVecs], wv[kGemvPrologueVecs];
+        static_assert(kGemvPrologueVecs == 8, "act_wait takes batches of eight");
+        float4_t xv[kGemvPrologueVecs], av[kGemvPrologueVecs], wv[kGemvPrologueVecs];
 #pragma unroll
-        for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = act_load4<kDev>(x4 + min(tid + j * kGemvThreads, n4 - 1));
+        for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(xv[j], x4 + min(tid + j * kGemvThreads, n4 - 1));
         if (a4 != nullptr) {
 #pragma unroll
-            for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + act_load4<kDev>(a4 + min(tid + j * kGemvThreads, n4 - 1)); // transformer.rs:442 / :445
+            for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(av[j], a4 + min(tid + j * kGemvThreads, n4 - 1));
         }
 #pragma unroll
         for (int j = 0; j < kGemvPrologueVecs; j++) wv[j] = w4[min(tid + j * kGemvThreads, n4 - 1)];
+        act_wait<kDevLoad>(xv);
+        if (a4 != nullptr) {
+            act_wait<kDevLoad>(av);
+#pragma unroll
+            for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + av[j]; // transformer.rs:442 / :445
+        }
         __builtin_amdgcn_sched_barrier(0);
         preload();
         float ss = 0.0f;
@@ -246,26 +284,32 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
         preload();
         float ss = 0.0f;
         for (int i = tid; i < K; i += kGemvThreads) {
-            float v = act_load1<kDev>(p.x + i);
-            if (p.x_add != nullptr) v = v + act_load1<kDev>(p.x_add + i);
+            float v = act_load1<kDevLoad>(p.x + i);
+            if (p.x_add != nullptr) v = v + act_load1<kDevLoad>(p.x_add + i);
             if (writes_sum) act_store1<kDev>(p.x_out + i, v);
             ss = fmaf(v, v, ss);
         }
         ss = block_sum(ss, red);
         const float rs = 1.0f / sqrtf(ss / (float)K + p.eps);
         for (int i = tid; i < K; i += kGemvThreads) {
-            float v = act_load1<kDev>(p.x + i);
-            if (p.x_add != nullptr) v = v + act_load1<kDev>(p.x_add + i);
+            float v = act_load1<kDevLoad>(p.x + i);
+            if (p.x_add != nullptr) v = v + act_load1<kDevLoad>(p.x_add + i);
             xs[i] = (XT)((v * rs) * p.norm_w[i]);
         }
     } else {
         for (int base = 0; base < n4; base += kGemvPrologueVecs * kGemvThreads) {
-            float4_t xv[kGemvPrologueVecs];
+            float4_t xv[kGemvPrologueVecs], av[kGemvPrologueVecs];
 #pragma unroll
-            for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = act_load4<kDev>(x4 + min(base + tid + j * kGemvThreads, n4 - 1));
+            for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(xv[j], x4 + min(base + tid + j * kGemvThreads, n4 - 1));
             if (a4 != nullptr) {
 #pragma unroll
-                for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + act_load4<kDev>(a4 + min(base + tid + j * kGemvThreads, n4 - 1));
+                for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(av[j], a4 + min(base + tid + j * kGemvThreads, n4 - 1));
+            }
+            act_wait<kDevLoad>(xv);
+            if (a4 != nullptr) {
+                act_wait<kDevLoad>(av);
+#pragma unroll
+                for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + av[j];
             }
             if (base == 0) {
                 __builtin_amdgcn_sched_barrier(0);
@@ -294,67 +338,72 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     //      grid reads one dense window of the matrix ----
     const int n_units = p.n_rows / kRows; // n_rows is a multiple of kRows (checked on the host)
     const int W = gridDim.x * kGemvWaves;
-
-    for (int unit = unit_first; unit < n_units; unit += W) {
-        const int row0 = unit * kRows;
-        float acc[kMats][kRows];
+    float acc[kMats][kRows];
+    auto clear_acc = [&]() {
 #pragma unroll
         for (int m = 0; m < kMats; m++)
 #pragma unroll
             for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
-
-        for (int c = 0; c < pieces; c += kU) {
-            uint4_t wv[kU][kMats][kRows];
-            if (kPre != kPreNone && have_pre && c == 0 && unit == unit_first) {
+    };
+    // the loads of the burst that starts at piece c of row unit `unit`
+    auto fetch = [&](int unit, int c, uint4_t (&wv)[kU][kMats][kRows]) {
+        const int row0 = unit * kRows;
+        if (c + kU <= pieces_full) {
+            // full burst: addresses differ by compile-time offsets
 #pragma unroll
-                for (int u = 0; u < kU; u++)
+            for (int u = 0; u < kU; u++)
 #pragma unroll
-                    for (int m = 0; m < kMats; m++)
+                for (int m = 0; m < kMats; m++)
 #pragma unroll
-                        for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[(u * kMats + m) * kRows + r];
-            } else if (c + kU <= pieces_full) {
-                // full burst: addresses differ by compile-time offsets
-#pragma unroll
-                for (int u = 0; u < kU; u++)
-#pragma unroll
-                    for (int m = 0; m < kMats; m++)
-#pragma unroll
-                        for (int r = 0; r < kRows; r++)
-                            wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + (size_t)(c + u) * kPiece + lane * kVec);
-            } else {
-                // tail burst: pieces past the end are skipped, the partial last piece is clamped to valid
-                // weights (they meet zeros of the padded x)
-#pragma unroll
-                for (int u = 0; u < kU; u++) {
-                    const int kk = min((c + u) * kPiece + lane * kVec, K - kVec);
-#pragma unroll
-                    for (int m = 0; m < kMats; m++)
-#pragma unroll
-                        for (int r = 0; r < kRows; r++) {
-                            if (c + u < pieces) wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + kk);
-                            else wv[u][m][r] = uint4_t{0u, 0u, 0u, 0u};
-                        }
-                }
-            }
+                    for (int r = 0; r < kRows; r++)
+                        wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + (size_t)(c + u) * kPiece + lane * kVec);
+        } else {
+            // tail burst: pieces past the end are skipped, the partial last piece is clamped to valid
+            // weights (they meet zeros of the padded x)
 #pragma unroll
             for (int u = 0; u < kU; u++) {
-                if (c + u < pieces) {
-                    float xv[kVec];
-                    load_x<XT, kVec>(xs + (c + u) * kPiece + lane * kVec, xv);
+                const int kk = min((c + u) * kPiece + lane * kVec, K - kVec);
 #pragma unroll
-                    for (int m = 0; m < kMats; m++)
+                for (int m = 0; m < kMats; m++)
 #pragma unroll
-                        for (int r = 0; r < kRows; r++) {
-                            float wf[kVec];
-                            WVec<WT>::unpack(wv[u][m][r], wf);
-#pragma unroll
-                            for (int i = 0; i < kVec; i++) acc[m][r] = fmaf(wf[i], xv[i], acc[m][r]);
-                        }
-                }
+                    for (int r = 0; r < kRows; r++) {
+                        if (c + u < pieces) wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + kk);
+                        else wv[u][m][r] = uint4_t{0u, 0u, 0u, 0u};
+                    }
             }
         }
-
-        // ---- reduce (valid in lane 63) and epilogue ----
+    };
+    auto take_pre = [&](auto dc, uint4_t (&wv)[kU][kMats][kRows]) {
+        constexpr int d = decltype(dc)::value;
+#pragma unroll
+        for (int u = 0; u < kU; u++)
+#pragma unroll
+            for (int m = 0; m < kMats; m++)
+#pragma unroll
+                for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[d][(u * kMats + m) * kRows + r];
+    };
+    // products of one burst against x from LDS
+    auto mac = [&](int c, const uint4_t (&wv)[kU][kMats][kRows]) {
+#pragma unroll
+        for (int u = 0; u < kU; u++) {
+            if (c + u < pieces) {
+                float xv[kVec];
+                load_x<XT, kVec>(xs + (c + u) * kPiece + lane * kVec, xv);
+#pragma unroll
+                for (int m = 0; m < kMats; m++)
+#pragma unroll
+                    for (int r = 0; r < kRows; r++) {
+                        float wf[kVec];
+                        WVec<WT>::unpack(wv[u][m][r], wf);
+#pragma unroll
+                        for (int i = 0; i < kVec; i++) acc[m][r] = fmaf(wf[i], xv[i], acc[m][r]);
+                    }
+            }
+        }
+    };
+    // reduce (valid in lane 63) and epilogue of one row unit
+    auto finish = [&](int unit) {
+        const int row0 = unit * kRows;
         float v[kMats][kRows];
 #pragma unroll
         for (int m = 0; m < kMats; m++)
@@ -400,6 +449,49 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
                     }
                 }
             }
+        }
+    };
+
+    if constexpr (kPre == kPreGiven) {
+        // The wavefront's bursts as one sequence, the first kD of them possibly already in registers (gemv_issue_bursts walks
+        // the same sequence).
+        int unit = unit_first, c = 0;
+        clear_acc();
+        auto advance = [&]() {
+            c += kU;
+            if (c >= pieces) {
+                finish(unit);
+                clear_acc();
+                c = 0;
+                unit += W;
+            }
+        };
+        static_for<kD>([&](auto dc) {
+            constexpr int d = decltype(dc)::value;
+            if (unit < n_units) {
+                uint4_t wv[kU][kMats][kRows];
+                if (pre_mask & (1u << d)) take_pre(dc, wv);
+                else fetch(unit, c, wv);
+                mac(c, wv);
+                advance();
+            }
+        });
+        while (unit < n_units) {
+            uint4_t wv[kU][kMats][kRows];
+            fetch(unit, c, wv);
+            mac(c, wv);
+            advance();
+        }
+    } else {
+        for (int unit = unit_first; unit < n_units; unit += W) {
+            clear_acc();
+            for (int c = 0; c < pieces; c += kU) {
+                uint4_t wv[kU][kMats][kRows];
+                if (kPre != kPreNone && (pre_mask & 1u) && c == 0 && unit == unit_first) take_pre(std::integral_constant<int, 0>{}, wv);
+                else fetch(unit, c, wv);
+                mac(c, wv);
+            }
+            finish(unit);
         }
     }
 }
