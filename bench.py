@@ -24,9 +24,11 @@ sys.path.insert(0, ROOT)
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per launch of the dominant kernel (c1: w13 GEMV; c3: w1-shape GEMM; 7B shapes) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs, each scaled by the same counter on a 1 GiB copy kernel (the PMC summary under profiles/ has the commands).
+# HBM bytes per launch of the dominant kernel (c1: w13 GEMV; c3: w1-shape GEMM; 7B shapes).  These are RECORDED values, not
+# something a bench run measures: they come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same script, each scaled
+# by the same counter on a 1 GiB copy kernel; the summaries named here hold the commands and the raw counter readings.
 MEASURED_TRAFFIC = {"c1": 181_001_730, "c3": 186_436_198}
+TRAFFIC_SOURCE = {"c1": "profiles/decode_c1_hbm_traffic_pmc.md", "c3": "profiles/prefill_c3_hbm_traffic_pmc.md"}
 
 CONFIGS = {
     # name: (dim, n_layers, n_heads, ffn_hidden, vocab, n_prompt, default decode steps)
@@ -70,20 +72,83 @@ def cpu_baseline(model, dim, n_layers, n_heads, ffn, vocab, n_prompt=8, n_decode
     t0 = time.perf_counter()
     logits = om.forward(toks, 0, oc)
     t_first = time.perf_counter() - t0
-    per = []
+    per, o_logits, o_ids = [], [logits], []
     for _ in range(n_decode):
         tok, _, _ = oracle.sample_greedy(logits)
         toks.append(tok)
+        o_ids.append(tok)
         t0 = time.perf_counter()
         logits = om.forward(toks[-1:], len(toks) - 1, oc)
         per.append(time.perf_counter() - t0)
+        o_logits.append(logits)
     ms = 1e3 * float(np.mean(per))
-    return {
+    baseline = {
         "value": round(ms, 2), "unit": "ms/token", "cores": cores, "kind": "port",
         "sample": f"same shape and weights, f16 mode, {n_prompt} prompt + {n_decode} greedy decode tokens "
                   f"(first call {1e3 * t_first:.0f} ms excluded)",
         "tokens_per_s": round(1e3 / ms, 3),
     }
+    # The same calls on the device (the oracle here is the checker, as in the tests): logits of every call against the
+    # oracle's, max |a - b| / max |b|, and the device's own greedy loop against the oracle's ids.
+    def rel(a, b):
+        return float(np.max(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64))) / max(float(np.max(np.abs(b))), 1e-30))
+    gc = model.make_caches()
+    errs = [rel(model.forward(prompt, 0, gc), o_logits[0])]
+    for i, tok in enumerate(o_ids):
+        errs.append(rel(model.forward([tok], n_prompt + i, gc), o_logits[i + 1]))
+    gc.free()
+    gc = model.make_caches()
+    g_ids, _, _ = model.generate_greedy(prompt, n_decode, gc)
+    gc.free()
+    same = 0
+    for a, b in zip(g_ids.tolist(), o_ids):
+        if a != b:
+            break
+        same += 1
+    parity = {"against": "CPU oracle (restatement of the reference's AVX2 path), full depth, same weights and token ids",
+              "max_rel_err": float(f"{max(errs):.3e}"), "tolerance": 1e-2, "measure": "max|a-b| / max|b| over the logits of each call",
+              "calls": len(errs), "greedy_ids_identical": same, "greedy_ids_compared": len(o_ids)}
+    return baseline, parity
+
+
+def measure_prefill(ra, ctx, model, prompt, reps, dim, n_layers, ffn, vocab):
+    """One forward over the whole prompt (+ the greedy pick): wall and HIP-event time to the first token, and the dominant
+    kernel -- the projection GEMM of the w1 / w3 shape (n x ffn x dim) -- timed alone with HIP events on the library's stream."""
+    n = len(prompt)
+    model.generate_greedy(prompt, 1, model.make_caches())            # warm-up (also sizes the work buffers)
+    times = []
+    for _ in range(reps):
+        cc = model.make_caches()
+        ctx.sync()
+        t0 = time.perf_counter()
+        _, ms_first, _ = model.generate_greedy(prompt, 1, cc)
+        ctx.sync()
+        times.append((1e3 * (time.perf_counter() - t0), ms_first))
+        cc.free()
+    wall_ms = float(np.mean([t[0] for t in times]))
+    ev_ms = float(np.mean([t[1] for t in times]))
+    flops_linear = 2.0 * n * n_layers * (4 * dim * dim + 3 * dim * ffn)
+    flops_attn = 2.0 * n * n * dim * n_layers          # causal: half of the dense 4 n^2 d
+    flops_head = 2.0 * vocab * dim
+    flops_total = flops_linear + flops_attn + flops_head
+    tflops = flops_total / (ev_ms * 1e-3) / 1e12
+    ga = ra.Tensor.from_numpy(ctx, ra.synth_normal_f16(1, 5, 0, n * dim, std=0.5).reshape(n, dim))
+    gb = ra.Tensor.from_numpy(ctx, ra.synth_normal_f16(2, 5, 0, ffn * dim, std=0.02).reshape(ffn, dim))
+    gc = ra.Tensor.zeros(ctx, n, ffn, ra.TensorDType.Float16)
+    for _ in range(3):
+        ra.check(ctx._lib.rlh_matrix_mul_inplace_transposed(gc._h, ga._h, gb._h))
+    ctx.sync()
+    iters = 20
+    e0 = ctx.event()
+    for _ in range(iters):
+        ra.check(ctx._lib.rlh_matrix_mul_inplace_transposed(gc._h, ga._h, gb._h))
+    e1 = ctx.event()
+    gemm_us = e0.elapsed_ms(e1) / iters * 1e3
+    gemm_flops = 2.0 * n * ffn * dim
+    gemm_tflops = gemm_flops / (gemm_us * 1e-6) / 1e12
+    for t in (ga, gb, gc):
+        t.free()
+    return wall_ms, ev_ms, tflops, gemm_us, gemm_tflops, gemm_flops, flops_total
 
 
 def bench_layer_split(args, ra, ctx, info) -> int:
@@ -143,6 +208,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill-block", action="store_true", help="c1: skip the 1024-token prefill measurement (prefill_c3)")
     ap.add_argument("--kernel-iters", type=int, default=320)
     ap.add_argument("--kernels-only", action="store_true",
                     help="skip the token loop and the CPU baseline: only the per-kernel timing loops (short runs for "
@@ -179,6 +245,11 @@ def main() -> int:
     K = args.steps if args.steps is not None else dflt_steps
     W = max(0, args.warmup)
     max_seq = max(n_prompt + max(K, W) + 1, (args.kernel_T or 0) + 1)
+    with_prefill_block = args.config == "c1" and not args.kernels_only and not args.no_prefill_block
+    if with_prefill_block:
+        max_seq = max(max_seq, 1025)   # room for the 1024-token prompt of the prefill block (config c3 on the same model)
+    if args.config == "c1" and not args.kernels_only:
+        max_seq = max(max_seq, 128 + 256 + 1)   # and for the full 128 + 256 workload when --steps asks for fewer
 
     ctx = ra.Context(0, verbose=False)
     info = ctx.device_info()
@@ -192,38 +263,11 @@ def main() -> int:
     if args.config == "c3":
         # prefill: time-to-first-token of one n_prompt-token forward (+ greedy pick), TFLOP/s against the dense f16 MFMA peak
         reps = max(1, K)
-        model.generate_greedy(prompt, 1, model.make_caches())            # warm-up (also sizes the work buffers)
-        times = []
-        for _ in range(reps):
-            cc = model.make_caches()
-            ctx.sync()
-            t0 = time.perf_counter()
-            _, ms_first, _ = model.generate_greedy(prompt, 1, cc)
-            ctx.sync()
-            times.append((1e3 * (time.perf_counter() - t0), ms_first))
-            cc.free()
-        wall_ms = float(np.mean([t[0] for t in times]))
-        ev_ms = float(np.mean([t[1] for t in times]))
         n = n_prompt
+        wall_ms, ev_ms, tflops, gemm_us, gemm_tflops, gemm_flops, flops_total = measure_prefill(ra, ctx, model, prompt, reps, dim, n_layers, ffn, vocab)
         flops_linear = 2.0 * n * n_layers * (4 * dim * dim + 3 * dim * ffn)
-        flops_attn = 2.0 * n * n * dim * n_layers          # causal: half of the dense 4 n^2 d
+        flops_attn = 2.0 * n * n * dim * n_layers
         flops_head = 2.0 * vocab * dim
-        tflops = (flops_linear + flops_attn + flops_head) / (ev_ms * 1e-3) / 1e12
-        # dominant kernel: the projection GEMM (w1 / w3 shape, n x ffn x dim), timed alone with HIP events on the library's stream
-        ga = ra.Tensor.from_numpy(ctx, ra.synth_normal_f16(1, 5, 0, n * dim, std=0.5).reshape(n, dim))
-        gb = ra.Tensor.from_numpy(ctx, ra.synth_normal_f16(2, 5, 0, ffn * dim, std=0.02).reshape(ffn, dim))
-        gc = ra.Tensor.zeros(ctx, n, ffn, ra.TensorDType.Float16)
-        for _ in range(3):
-            ra.check(ctx._lib.rlh_matrix_mul_inplace_transposed(gc._h, ga._h, gb._h))
-        ctx.sync()
-        iters = 20
-        e0 = ctx.event()
-        for _ in range(iters):
-            ra.check(ctx._lib.rlh_matrix_mul_inplace_transposed(gc._h, ga._h, gb._h))
-        e1 = ctx.event()
-        gemm_us = e0.elapsed_ms(e1) / iters * 1e3
-        gemm_flops = 2.0 * n * ffn * dim
-        gemm_tflops = gemm_flops / (gemm_us * 1e-6) / 1e12
         out = {
             "metric": "time to first token, LLaMA-7B-shape f16 prompt prefill (1024 tokens), 1 MI355X",
             "value": round(wall_ms, 3), "unit": "ms", "n_gpus": 1, "steps": reps, "warmup": 1, "ms_per_step": round(wall_ms, 3),
@@ -234,6 +278,7 @@ def main() -> int:
             "tflops_end_to_end": round(tflops, 1), "algorithmic_flops_end_to_end": flops_linear + flops_attn + flops_head,
             "roofline": {"bound": "mfma", "kernel": f"gemm_f16_dma_kernel (256x192 tile, v_mfma_f32_32x32x16_f16) on the w1/w3 product {n}x{ffn}x{dim}",
                          "achieved": round(gemm_tflops, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(gemm_tflops / 2500.0, 4), "traffic": MEASURED_TRAFFIC.get("c3"),
+                         "traffic_source": TRAFFIC_SOURCE["c3"] + " (recorded rocprofv3 --pmc run, not measured by this run)",
                          "us_per_launch": round(gemm_us, 2), "algorithmic_flops": gemm_flops,
                          "algorithmic_bytes_per_launch": 2 * (n * dim + ffn * dim + n * ffn)},
             "cpu_baseline": None, "device": info["name"],
@@ -290,6 +335,7 @@ def main() -> int:
         "bound": "hbm", "kernel": "gemv_kernel<f16 weights, f16 x, SiLU epilogue> (" + dom + ")",
         "achieved": kernels[dom]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(kernels[dom]["GBps"] / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC.get(args.config),
+        "traffic_source": (TRAFFIC_SOURCE[args.config] + " (recorded rocprofv3 --pmc run, not measured by this run)") if args.config in TRAFFIC_SOURCE else None,
         "algorithmic_bytes_per_launch": kernels[dom]["bytes"], "us_per_launch": kernels[dom]["us"],
     }
 
@@ -320,8 +366,34 @@ def main() -> int:
         "device": info["name"],
         "first_tokens": [int(first_ids[0])] + [int(t) for t in ids[:7]],
     }
+    if args.config == "c1" and K != dflt_steps:
+        # the benchmark definition's workload is 128 prompt + 256 decode tokens; with another --steps the line above is quoted on
+        # a shorter (or longer) sequence, so the full workload is measured too
+        c2 = model.make_caches()
+        model.generate_greedy(prompt, 1, c2)
+        ctx.sync()
+        t0 = time.perf_counter()
+        model.decode_greedy(dflt_steps, c2)
+        ctx.sync()
+        ms256 = 1e3 * (time.perf_counter() - t0) / dflt_steps
+        b256 = float(np.mean([model.decode_bytes(n_prompt + i + 1) for i in range(dflt_steps)]))
+        out["workload_128_plus_256"] = {"ms_per_token": round(ms256, 4), "hbm_frac_end_to_end": round(b256 / (ms256 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                        "note": f"--steps {K} changes the mean sequence length; this is the defined workload (256 decode steps)"}
+        c2.free()
+    if with_prefill_block:
+        # config c3 on the same weights: one forward over a 1024-token prompt, MFMA roofline of its dominant GEMM
+        p1024 = ra.synth_tokens(0, 1024, 3, vocab)
+        wall_p, ev_p, tflops_p, gemm_us, gemm_tflops, gemm_flops, flops_total = measure_prefill(ra, ctx, model, p1024, 3, dim, n_layers, ffn, vocab)
+        out["prefill_c3"] = {
+            "workload": "c3: one forward over a 1024-token prompt on the same model", "ttft_ms": round(wall_p, 3), "ttft_ms_hip_events": round(ev_p, 3),
+            "prompt_tokens_per_s": round(1024 / (wall_p * 1e-3), 1), "tflops_end_to_end": round(tflops_p, 1), "algorithmic_flops_end_to_end": flops_total,
+            "roofline": {"bound": "mfma", "kernel": f"gemm_f16_dma_kernel (256x192 tile, v_mfma_f32_32x32x16_f16) on the w1/w3 product 1024x{ffn}x{dim}",
+                         "achieved": round(gemm_tflops, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(gemm_tflops / 2500.0, 4),
+                         "us_per_launch": round(gemm_us, 2), "algorithmic_flops": gemm_flops, "traffic": MEASURED_TRAFFIC["c3"],
+                         "traffic_source": TRAFFIC_SOURCE["c3"] + " (recorded rocprofv3 --pmc run, not measured by this run)"},
+        }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(model, dim, n_layers, n_heads, ffn, vocab)
+        out["cpu_baseline"], out["parity"] = cpu_baseline(model, dim, n_layers, n_heads, ffn, vocab)
     else:
         out["cpu_baseline"] = None
     caches.free()
