@@ -1048,9 +1048,27 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         normed = 0;
         if ((rc = gemm(S.a, d, L.wo.p, d, S.h, d, n, d, d, kGemmEpiResAddF32, S.x, nullptr, (const float *)L.ffn_norm.p, &normed)) != RLH_OK) return rc; // h = x + wo(att)
         if (!normed) HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.h, (const float *)L.ffn_norm.p, n, d, eps, st));
-        if ((rc = gemm(S.xn, d, L.w1.p, d, S.g, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
-        // w3's epilogue applies SiLU(w1 x) * (w3 x) and the f16 rounding points of transformer.rs:557-565 in place of a pass of its own
-        if ((rc = gemm(S.xn, d, L.w3.p, d, S.mm, F, n, F, d, kGemmEpiSiluGateF16, nullptr, S.g)) != RLH_OK) return rc;
+        {
+            // SiLU(w1 x) * (w3 x) with the f16 rounding points of transformer.rs:557-565: where the shape allows, both products
+            // in one pass over xn; otherwise w1's product goes to memory and w3's epilogue consumes it
+            GemmParams g{};
+            g.a = (const _Float16 *)S.xn;
+            g.b = (const _Float16 *)L.w1.p;
+            g.b2 = (const _Float16 *)L.w3.p;
+            g.c = S.mm;
+            g.m = n;
+            g.n = F;
+            g.k = d;
+            g.lda = g.ldb = d;
+            g.ldc = F;
+            g.batch = 1;
+            if (gemm_f16_dual_gate_supported(g)) {
+                HIP_TRY(launch_gemm_f16(g, kGemmEpiSiluGateF16, st));
+            } else {
+                if ((rc = gemm(S.xn, d, L.w1.p, d, S.g, F, n, F, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
+                if ((rc = gemm(S.xn, d, L.w3.p, d, S.mm, F, n, F, d, kGemmEpiSiluGateF16, nullptr, S.g)) != RLH_OK) return rc;
+            }
+        }
         // x = h + w2(...); the next block's attention_norm rides along where it can
         normed = 0;
         const float *next_norm = l < l_last ? (const float *)m->layers[(size_t)l + 1].attn_norm.p : nullptr;

@@ -255,7 +255,7 @@ __global__ __launch_bounds__(kApThreads, 2) void attn_prefill_kernel(AttnPrefill
             for (int g = 0; g < 4; g++) {
                 half4_t o;
 #pragma unroll
-                for (int i = 0; i < 4; i++) o[i] = (half_t)(o_acc[d][g * 4 + i] * inv0 + mb[(d * 16 + g * 4 + i) * 64] * inv1);
+                for (int i = 0; i < 4; i++) o[i] = to_f16(o_acc[d][g * 4 + i] * inv0 + mb[(d * 16 + g * 4 + i) * 64] * inv1);
                 *reinterpret_cast<half4_t *>(ot + col * kOutRowHalves + d * 32 + g * 8 + half * 4) = o;
             }
         // rows q0 .. q0 + 31, columns head * HD .. + HD of wo's input

@@ -16,7 +16,16 @@ constexpr int kWave = 64;
 
 // f32 -> f16 -> f32 with round-to-nearest-even: the reference's rounding points
 // (half::f16::from_f32 / _mm256_cvtps_ph(a, 0), simd_support.rs:50-52, tensor.rs:374-375).
-__device__ __forceinline__ float f16r(float v) { return (float)(half_t)v; }
+// The conversion goes through as_f32: left to itself hipcc folds an f32 multiply (or multiply-add) whose only use is a conversion
+// to f16 into v_fma_mixlo_f16, which rounds the exact product once, to f16, where the reference rounds it to f32 first and to
+// f16 after; the two differ for about 6 products in 100000 (counted on the part over 2^24 random pairs).  An empty asm
+// statement keeps the value a plain f32 register.
+__device__ __forceinline__ float as_f32(float v) {
+    asm("" : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ half_t to_f16(float v) { return (half_t)as_f32(v); }
+__device__ __forceinline__ float f16r(float v) { return (float)to_f16(v); }
 
 // ---- DPP cross-lane moves (GFX9 encodings) -------------------------------------------------
 constexpr int kDppQuadPerm1032 = 0xB1;   // lanes i <-> i^1
@@ -120,6 +129,12 @@ __device__ __forceinline__ float silu_fast(float v) {
 // here the waits are placed by hand (vmcnt is decremented in issue order).
 __device__ __forceinline__ void dma16(const half_t *src, unsigned dst) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory");
+}
+
+// The same with the address as a wave-uniform base (scalar registers) plus a 32-bit byte offset per lane: half the vector
+// registers per load address of the form above.
+__device__ __forceinline__ void dma16_base(const half_t *base, unsigned byte_off, unsigned dst) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(dst) : "memory");
 }
 
 template <int kN>

@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_f16_kernel(GemmParams p) {
                         *cp = p.accumulate ? (*cp + val) : val;
                     } else if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
                         const float g = (float)p.gate[(size_t)r * p.ldc + c];
-                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)(silu_fast(g) * f16r(val));
+                        reinterpret_cast<half_t *>(p.c)[off] = to_f16(silu_fast(g) * f16r(val));
                     } else { // kGemmEpiResAddF32: residual add of transformer.rs:442 / :445 on the f16-rounded product
                         reinterpret_cast<float *>(p.c)[off] = p.residual[(size_t)r * p.ldc + c] + f16r(val);
                     }
@@ -135,6 +135,7 @@ hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s) {
         return launch_gemm_f16_dma(p, epilogue, s);
     }
     if (p.m <= 0 || p.n <= 0 || p.k <= 0 || (p.k % 8) != 0 || (p.lda % 8) != 0 || (p.ldb % 8) != 0 || p.batch < 1) return hipErrorInvalidValue;
+    if (p.b2 != nullptr) return gemm_f16_dual_gate_supported(p) ? launch_gemm_f16_dma(p, epilogue, s) : hipErrorInvalidValue; // fast path only
     // RLLAMA_HIP_GEMM_SIMPLE=1 keeps every product on the kernel of this file (tuning / cross-checks)
     static const bool simple_only = getenv("RLLAMA_HIP_GEMM_SIMPLE") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_SIMPLE")) != 0;
     if (p.k_seg != 0 || p.causal != 0) return gemm_f16_dma_supported(p) ? launch_gemm_f16_dma(p, epilogue, s) : hipErrorInvalidValue;

@@ -32,8 +32,14 @@ typedef __attribute__((ext_vector_type(16))) float float16_t;
 // with a row of kBK / 2 floats; a 16-byte fragment then holds 4 consecutive k of a row and feeds 4
 // v_mfma_f32_32x32x2_f32 (k slot of lane half h in the j-th of them: float j of chunk 2 ks + h, for A and B alike).
 // kIT: 32-row MFMA tiles per wavefront (2: wavefronts of 64 x 32 kNT; 1: 32 x 32 kNT, for products with at most 32 rows).
-template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false, int kIT = 2>
+// kDual: two products of the same A in one pass -- A * B^T and A * B2^T (w1 and w3 of the feed-forward block,
+// transformer.rs:551-565) -- with two accumulator sets per wavefront: a K-tile of A is staged once for both, so the L2 -> LDS
+// bytes per flop fall by a further 29 % on the 256 x 192 tile, the gate never goes to memory and comes back, and the
+// epilogue writes SiLU(f16(A B^T)) * f16(A B2^T) straight from the accumulators.
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false, int kIT = 2, bool kDual = false>
 __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams p) {
+    static_assert(!kDual || (kEpi == kGemmEpiSiluGateF16 && !kF32), "two products share the SiLU-gate epilogue only");
+    constexpr int kP = kDual ? 2 : 1;                    // products
     constexpr int kE = kF32 ? 2 : 1;                     // halves per operand element: k, lda, ldb, strides count elements
     constexpr int kWaves = 2 * kWavesM;
     constexpr int kWR = 32 * kIT;                        // rows of a wavefront's tile
@@ -42,7 +48,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     constexpr int kRowsPerLoad = 64 / kCpr;              // rows one wavefront-wide load covers (1 KiB of LDS)
     constexpr int kSwzDiv = 16 / kCpr;                   // physical chunk = logical chunk ^ ((row / kSwzDiv) % kCpr)
     constexpr int kRowBytes = kBK * 2;
-    constexpr int kStageBytes = (kBM + kBN) * kRowBytes;
+    constexpr int kStageBytes = (kBM + kP * kBN) * kRowBytes;
     constexpr int kGroups = kStageBytes / 1024;          // 1 KiB row groups per stage, dealt round-robin to wavefronts
     constexpr int kLoadsMax = (kGroups + kWaves - 1) / kWaves;
     constexpr int kLoadsMin = kGroups / kWaves;
@@ -95,13 +101,15 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
     for (int i = 0; i < kLoadsMax; i++) {
         const int g = min(i * kWaves + wave, kGroups - 1);
-        const int row2 = g * kRowsPerLoad + l_row;       // 0 .. kBM + kBN - 1 over A then B
+        const int row2 = g * kRowsPerLoad + l_row;       // 0 .. kBM + kP kBN - 1 over A, then B (, then B2)
         const bool is_b = row2 >= kBM;
-        const int row = is_b ? row2 - kBM : row2;
+        const bool is_b2 = kDual && row2 >= kBM + kBN;
+        const int row = is_b2 ? row2 - kBM - kBN : is_b ? row2 - kBM : row2;
         const int lc = l_pc ^ ((row / kSwzDiv) % kCpr);  // logical chunk this lane fetches
         // rows past the matrix edge are clamped to a valid row; what they produce is never stored
         const int grow = is_b ? min(bn0 + row, N - 1) : min(bm0 + row, M - 1);
-        gsrc[i] = (is_b ? B + (size_t)grow * p.ldb * kE : A + (size_t)grow * p.lda * kE) + lc * 8;
+        const half_t *bsrc = is_b2 ? p.b2 : B;
+        gsrc[i] = (is_b ? bsrc + (size_t)grow * p.ldb * kE : A + (size_t)grow * p.lda * kE) + lc * 8;
         src_is_b[i] = is_b;
     }
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_raw;
@@ -123,11 +131,12 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         }
     };
 
-    float16_t acc[kIT][kNT];
+    constexpr int kNTs = kP * kNT;                       // column tiles of a wavefront over all products (product q: j / kNT)
+    float16_t acc[kIT][kNTs];
 #pragma unroll
     for (int i = 0; i < kIT; i++)
 #pragma unroll
-        for (int j = 0; j < kNT; j++)
+        for (int j = 0; j < kNTs; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
@@ -153,8 +162,8 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // SiLU-gate epilogue: the gate values this lane will need (the 16-byte pieces it handles in the row-wise epilogue below)
     // are fetched now as well, for the same reason.
     [[maybe_unused]] const bool rows16 = (p.ldc % 8) == 0 && (N % 8) == 0 && ((zb * p.stride_c) % 8) == 0 && (reinterpret_cast<uintptr_t>(p.c) % 16) == 0 &&
-                                         (kEpi != kGemmEpiSiluGateF16 || (reinterpret_cast<uintptr_t>(p.gate) % 16) == 0);
-    constexpr bool kGatePre = kEpi == kGemmEpiSiluGateF16 && kNT * kIT <= 6; // the widest tile has no registers to spare for it
+                                         (kEpi != kGemmEpiSiluGateF16 || kDual || (reinterpret_cast<uintptr_t>(p.gate) % 16) == 0);
+    constexpr bool kGatePre = kEpi == kGemmEpiSiluGateF16 && !kDual && kNT * kIT <= 6; // the widest tile has no registers to spare for it
     constexpr int kRowChunks = 32 * kNT / 8;             // 16-byte pieces per row of a wavefront's tile
     constexpr int kGateChunks = kGatePre ? kRowChunks * kWR / 64 : 1;
     [[maybe_unused]] half8_t gate_pre[kGateChunks];
@@ -172,7 +181,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 
     // operand fragments: lane l supplies row (l % 32), logical chunk 2 * ks + l / 32 of a 32 x 16 slab
     const int frow = lane & 31, fch = lane >> 5;
-    int a_off[kIT], a_sw[kIT], b_off[kNT], b_sw[kNT];
+    int a_off[kIT], a_sw[kIT], b_off[kNTs], b_sw[kNTs];
 #pragma unroll
     for (int i = 0; i < kIT; i++) {
         const int ra = wm * kWR + i * 32 + frow;
@@ -180,9 +189,9 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         a_sw[i] = (ra / kSwzDiv) % kCpr;
     }
 #pragma unroll
-    for (int j = 0; j < kNT; j++) {
-        const int rb = wn * (32 * kNT) + j * 32 + frow;
-        b_off[j] = (kBM + rb) * kRowBytes;
+    for (int j = 0; j < kNTs; j++) {
+        const int rb = wn * (32 * kNT) + (j % kNT) * 32 + frow; // row within its own matrix (the swizzle counts from there)
+        b_off[j] = (kBM + (j / kNT) * kBN + rb) * kRowBytes;
         b_sw[j] = (rb / kSwzDiv) % kCpr;
     }
 
@@ -192,9 +201,10 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // of K-step s run (two fragment sets, selected by the parity of the unrolled K-step); the tile change sits in
     // the middle of the last K-step's MFMAs so that the barrier and the LDS latency behind it stay covered.
     constexpr int kKS = kBK / 16;
-    constexpr int kSplitJ = kNT / 2; // column tiles of the last K-step whose MFMAs run before the tile change (0 .. kNT measured alike)
+    constexpr int kSplitJ = kNTs / 2; // column tiles of the last K-step whose MFMAs run before the tile change (0 .. kNT measured alike)
     static_assert(kKS % 2 == 0, "fragment sets alternate by K-step parity");
-    half8_t af[2][kIT], bf[2][kNT];
+    half8_t af[2][kIT];
+    [[maybe_unused]] half8_t bf[2][kDual ? 1 : kNT];
     auto mma = [&](const half8_t &a, const half8_t &b, float16_t &c) {
         if constexpr (kF32) {
             const float4_t a4 = __builtin_bit_cast(float4_t, a), b4 = __builtin_bit_cast(float4_t, b);
@@ -209,54 +219,154 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
 #pragma unroll
         for (int i = 0; i < kIT; i++) af[set][i] = *reinterpret_cast<const half8_t *>(stage + a_off[i] + ((lc ^ a_sw[i]) << 4));
 #pragma unroll
-        for (int j = 0; j < kNT; j++) bf[set][j] = *reinterpret_cast<const half8_t *>(stage + b_off[j] + ((lc ^ b_sw[j]) << 4));
+        for (int j = 0; j < (kDual ? 0 : kNT); j++) bf[set][j] = *reinterpret_cast<const half8_t *>(stage + b_off[j] + ((lc ^ b_sw[j]) << 4));
     };
+    if constexpr (kDual) {
+        // Two products: 192 accumulator registers of the 256 a wavefront has here, so everything else is kept small.  Staging
+        // addresses are a uniform base per matrix (tile origin + k, scalar registers) plus one 32-bit offset per load that B and
+        // B2 share; B fragments are single-buffered per product -- those of product 1 are read while the MFMAs of product 0 run,
+        // those of product 0 for the next K-step (with A's, double-buffered) while product 1's run.
+        static_assert((kBM / kRowsPerLoad) % kWaves == 0 && (kBN / kRowsPerLoad) % kWaves == 0, "every load of a wavefront stays within one matrix");
+        static_assert(kSwzDiv * kCpr <= 32 && 32 % (kSwzDiv * kCpr) == 0, "one swizzle term for all fragments of a lane");
+        constexpr int kLA = kBM / kRowsPerLoad / kWaves, kLB = kBN / kRowsPerLoad / kWaves;
+        constexpr int kLoads = kLA + 2 * kLB;
+        unsigned voff_a[kLA], voff_b[kLB];
 #pragma unroll
-    for (int t = 0; t < kStages; t++) issue(t);
-    if (short_wave) wait_vmcnt<(kStages - 1) * kLoadsMin>();
-    else wait_vmcnt<(kStages - 1) * kLoadsMax>();
-    __syncthreads();
-    read_frags(0, lds_raw, 0);
-    for (int kt = 0; kt < n_kt; kt++) {
-        const unsigned char *stage = lds_raw + (kt % kStages) * kStageBytes;
+        for (int i = 0; i < kLA; i++) {
+            const int row = (i * kWaves + wave) * kRowsPerLoad + l_row;
+            const int lc = l_pc ^ ((row / kSwzDiv) % kCpr);
+            voff_a[i] = (unsigned)(((min(bm0 + row, M - 1) - bm0) * p.lda + lc * 8) * 2);
+        }
 #pragma unroll
-        for (int ks = 0; ks < kKS; ks++) {
-            const int cur = ks & 1, nxt = cur ^ 1;
-            if (ks + 1 < kKS) {
-                read_frags(nxt, stage, ks + 1);
+        for (int i = 0; i < kLB; i++) {
+            const int row = (i * kWaves + wave) * kRowsPerLoad + l_row;
+            const int lc = l_pc ^ ((row / kSwzDiv) % kCpr);
+            voff_b[i] = (unsigned)(((min(bn0 + row, N - 1) - bn0) * p.ldb + lc * 8) * 2);
+        }
+        const half_t *s_a = A + (size_t)bm0 * p.lda, *s_b = B + (size_t)bn0 * p.ldb, *s_b2 = p.b2 + (size_t)bn0 * p.ldb;
+        int iss_k = 0;
+        auto issue2 = [&](int kt) {
+            const unsigned dst = lds_base + (unsigned)(kt % kStages) * kStageBytes + (unsigned)wave * 1024;
+#pragma unroll
+            for (int i = 0; i < kLA; i++) dma16_base(s_a + iss_k, voff_a[i], dst + i * (kWaves * 1024));
+#pragma unroll
+            for (int i = 0; i < kLB; i++) dma16_base(s_b + iss_k, voff_b[i], dst + (kLA + i) * (kWaves * 1024));
+#pragma unroll
+            for (int i = 0; i < kLB; i++) dma16_base(s_b2 + iss_k, voff_b[i], dst + (kLA + kLB + i) * (kWaves * 1024));
+            if (kt + 1 < n_kt) iss_k += kBK; // past the end the last tile is loaded again (keeps the in-flight count constant)
+        };
+        const int sw = (frow / kSwzDiv) % kCpr;
+        const int xa = (wm * kWR + frow) * kRowBytes, xb = (kBM + wn * (32 * kNT) + frow) * kRowBytes;
+        half8_t b0[kNT], b1[kNT];
+        auto read_a = [&](int set, const unsigned char *stage, int ks) {
+            const int c = ((ks * 2 + fch) ^ sw) << 4;
+#pragma unroll
+            for (int i = 0; i < kIT; i++) af[set][i] = *reinterpret_cast<const half8_t *>(stage + xa + i * (32 * kRowBytes) + c);
+        };
+        auto read_b = [&](half8_t (&b)[kNT], const unsigned char *stage, int ks, int q) {
+            const int c = ((ks * 2 + fch) ^ sw) << 4;
+#pragma unroll
+            for (int j = 0; j < kNT; j++) b[j] = *reinterpret_cast<const half8_t *>(stage + xb + (q * kBN + j * 32) * kRowBytes + c);
+        };
+#pragma unroll
+        for (int t = 0; t < kStages; t++) issue2(t);
+        wait_vmcnt<(kStages - 1) * kLoads>();
+        __syncthreads();
+        read_a(0, lds_raw, 0);
+        read_b(b0, lds_raw, 0, 0);
+        for (int kt = 0; kt < n_kt; kt++) {
+            const unsigned char *stage = lds_raw + (kt % kStages) * kStageBytes;
+#pragma unroll
+            for (int ks = 0; ks < kKS; ks++) {
+                const int cur = ks & 1, nxt = cur ^ 1;
+                read_b(b1, stage, ks, 1);
 #pragma unroll
                 for (int j = 0; j < kNT; j++)
 #pragma unroll
-                    for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
-                {   // order within the step: an LDS fragment read of the next step behind each of the first MFMAs of this one,
-                    // so that the reads are in flight under the matrix pipe and none is left to wait for when the next step
-                    // begins (left to itself the scheduler issues the reads at the end of the step and the MFMAs wait for them)
-                    constexpr int kPerMma = kF32 ? 4 : 1; // MFMA instructions per fragment pair
-                    constexpr int kMmas = kIT * kNT, kReads = kIT + kNT, kPairs = kMmas < kReads ? kMmas : kReads;
+                    for (int i = 0; i < kIT; i++) mma(af[cur][i], b0[j], acc[i][j]);
 #pragma unroll
-                    for (int r = 0; r < kPairs; r++) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, kPerMma, 0); // MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // DS read
-                    }
-                    if constexpr (kMmas > kPairs) __builtin_amdgcn_sched_group_barrier(0x008, (kMmas - kPairs) * kPerMma, 0);
-                    if constexpr (kReads > kPairs) __builtin_amdgcn_sched_group_barrier(0x100, kReads - kPairs, 0);
+                for (int r = 0; r < kNT; r++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
                 }
-            } else {
+                __builtin_amdgcn_sched_group_barrier(0x008, kIT * kNT - kNT, 0);
+                if (ks + 1 < kKS) {
+                    read_a(nxt, stage, ks + 1);
+                    read_b(b0, stage, ks + 1, 0);
 #pragma unroll
-                for (int j = 0; j < kSplitJ; j++)
+                    for (int j = 0; j < kNT; j++)
 #pragma unroll
-                    for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
-                __builtin_amdgcn_sched_barrier(0);
-                if (short_wave) wait_vmcnt<(kStages - 2) * kLoadsMin>();
-                else wait_vmcnt<(kStages - 2) * kLoadsMax>();
-                __syncthreads(); // K-tile kt + 1 is in LDS for everybody, and nobody reads K-tile kt any more
-                issue(kt + kStages);
-                read_frags(nxt, lds_raw + ((kt + 1) % kStages) * kStageBytes, 0);
-                __builtin_amdgcn_sched_barrier(0);
+                        for (int i = 0; i < kIT; i++) mma(af[cur][i], b1[j], acc[i][kNT + j]);
 #pragma unroll
-                for (int j = kSplitJ; j < kNT; j++)
+                    for (int r = 0; r < kIT + kNT; r++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, kIT * kNT - (kIT + kNT), 0);
+                } else {
+                    __builtin_amdgcn_sched_barrier(0);
+                    wait_vmcnt<(kStages - 2) * kLoads>();
+                    __syncthreads(); // K-tile kt + 1 is in LDS for everybody, and nobody reads K-tile kt any more
+                    issue2(kt + kStages);
+                    const unsigned char *next = lds_raw + ((kt + 1) % kStages) * kStageBytes;
+                    read_a(nxt, next, 0);
+                    read_b(b0, next, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                    for (int j = 0; j < kNT; j++)
+#pragma unroll
+                        for (int i = 0; i < kIT; i++) mma(af[cur][i], b1[j], acc[i][kNT + j]);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < kStages; t++) issue(t);
+        if (short_wave) wait_vmcnt<(kStages - 1) * kLoadsMin>();
+        else wait_vmcnt<(kStages - 1) * kLoadsMax>();
+        __syncthreads();
+        read_frags(0, lds_raw, 0);
+        for (int kt = 0; kt < n_kt; kt++) {
+            const unsigned char *stage = lds_raw + (kt % kStages) * kStageBytes;
+#pragma unroll
+            for (int ks = 0; ks < kKS; ks++) {
+                const int cur = ks & 1, nxt = cur ^ 1;
+                if (ks + 1 < kKS) {
+                    read_frags(nxt, stage, ks + 1);
+#pragma unroll
+                    for (int j = 0; j < kNTs; j++)
+#pragma unroll
+                        for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                    {   // order within the step: an LDS fragment read of the next step behind each of the first MFMAs of this one,
+                        // so that the reads are in flight under the matrix pipe and none is left to wait for when the next step
+                        // begins (left to itself the scheduler issues the reads at the end of the step and the MFMAs wait for them)
+                        constexpr int kPerMma = kF32 ? 4 : 1; // MFMA instructions per fragment pair
+                        constexpr int kMmas = kIT * kNTs, kReads = kIT + kNTs, kPairs = kMmas < kReads ? kMmas : kReads;
+#pragma unroll
+                        for (int r = 0; r < kPairs; r++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, kPerMma, 0); // MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // DS read
+                        }
+                        if constexpr (kMmas > kPairs) __builtin_amdgcn_sched_group_barrier(0x008, (kMmas - kPairs) * kPerMma, 0);
+                        if constexpr (kReads > kPairs) __builtin_amdgcn_sched_group_barrier(0x100, kReads - kPairs, 0);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < kSplitJ; j++)
+#pragma unroll
+                        for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (short_wave) wait_vmcnt<(kStages - 2) * kLoadsMin>();
+                    else wait_vmcnt<(kStages - 2) * kLoadsMax>();
+                    __syncthreads(); // K-tile kt + 1 is in LDS for everybody, and nobody reads K-tile kt any more
+                    issue(kt + kStages);
+                    read_frags(nxt, lds_raw + ((kt + 1) % kStages) * kStageBytes, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int j = kSplitJ; j < kNTs; j++)
+#pragma unroll
+                        for (int i = 0; i < kIT; i++) mma(af[cur][i], bf[cur][j], acc[i][j]);
+                }
             }
         }
     }
@@ -285,7 +395,11 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                 for (int j = 0; j < kNT; j++)
 #pragma unroll
                     for (int v = 0; v < 16; v++)
-                        tile[(i * 32 + (v >> 2) * 8 + row_in + (v & 3)) * kTS + j * 32 + col_in] = (half_t)acc[i][j][v]; // tensor.rs:1623-1643
+                    {
+                        half_t o = (half_t)acc[i][j][v]; // tensor.rs:1623-1643
+                        if constexpr (kDual) o = to_f16(silu_fast(f16r(acc[i][j][v])) * f16r(acc[i][kNT + j][v])); // tensor.rs:822-832 on the f16 gate
+                        tile[(i * 32 + (v >> 2) * 8 + row_in + (v & 3)) * kTS + j * 32 + col_in] = o;
+                    }
             half_t *cbase = reinterpret_cast<half_t *>(p.c) + zb * p.stride_c;
 #pragma unroll
             for (int it = 0; it < kChunks * kWR / 64; it++) {
@@ -295,14 +409,14 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                 if (r < M && c < N) {
                     half8_t o = *reinterpret_cast<const half8_t *>(tile + rr * kTS + ch * 8);
                     const size_t off = (size_t)r * p.ldc + c;
-                    if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
+                    if constexpr (kEpi == kGemmEpiSiluGateF16 && !kDual) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
                         half8_t g8;
                         if constexpr (kGatePre) g8 = gate_pre[it];
                         else g8 = *reinterpret_cast<const half8_t *>(p.gate + off);
 #pragma unroll
                         for (int e = 0; e < 8; e++) {
                             const float g = (float)g8[e];
-                            o[e] = (half_t)(silu_fast(g) * (float)o[e]);
+                            o[e] = to_f16(silu_fast(g) * (float)o[e]);
                         }
                     }
                     *reinterpret_cast<half8_t *>(cbase + off) = o;
@@ -323,6 +437,11 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         if constexpr (kEarlyResidual) {
 #pragma unroll
             for (int i = 0; i < kIT; i++) prev[i] = early[i][j];
+        } else if constexpr (kDual) {
+#pragma unroll
+            for (int i = 0; i < kIT; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) prev[i][v] = f16r(acc[i][j][v]);
         } else if constexpr (kEpi == kGemmEpiSiluGateF16) {
 #pragma unroll
             for (int i = 0; i < kIT; i++)
@@ -346,7 +465,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
             for (int v = 0; v < 16; v++) {
                 const int r = out_row(i, v);
                 if (r < M && c < N) {
-                    const float val = acc[i][j][v];
+                    const float val = acc[i][kDual ? kNT + j : j][v];
                     const size_t off = zb * p.stride_c + (size_t)r * p.ldc + c;
                     if constexpr (kEpi == kGemmEpiF16) {
                         reinterpret_cast<half_t *>(p.c)[off] = (half_t)val; // tensor.rs:1623-1643
@@ -354,7 +473,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                         reinterpret_cast<float *>(p.c)[off] = prev[i][v] + val;
                     } else if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
                         const float g = prev[i][v];
-                        reinterpret_cast<half_t *>(p.c)[off] = (half_t)(silu_fast(g) * f16r(val));
+                        reinterpret_cast<half_t *>(p.c)[off] = to_f16(silu_fast(g) * f16r(val));
                     } else { // kGemmEpiResAddF32: residual add of transformer.rs:442 / :445 on the f16-rounded product
                         reinterpret_cast<float *>(p.c)[off] = prev[i][v] + f16r(val);
                     }
@@ -372,16 +491,16 @@ bool gemm_f16_dma_supported(const GemmParams &p) {
     return p.causal >= 0 && p.causal <= 2;
 }
 
-template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false, int kIT = 2>
+template <int kEpi, int kWavesM, int kNT, int kBK, int kStages, bool kF32 = false, int kIT = 2, bool kDual = false>
 static hipError_t launch_dma(const GemmParams &p, hipStream_t s) {
     constexpr int bm = 32 * kIT * kWavesM, bn = 64 * kNT;
-    constexpr size_t lds = (size_t)kStages * (bm + bn) * kBK * 2;
+    constexpr size_t lds = (size_t)kStages * (bm + (kDual ? 2 : 1) * bn) * kBK * 2;
     static_assert(lds <= 160 * 1024, "LDS of one compute unit");
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32, kIT>),
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32, kIT, kDual>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) return attr;
     dim3 grid((p.n + bn - 1) / bn, (p.m + bm - 1) / bm, p.batch);
-    hipLaunchKernelGGL((gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32, kIT>), grid, dim3(128 * kWavesM), lds, s, p);
+    hipLaunchKernelGGL((gemm_f16_dma_kernel<kEpi, kWavesM, kNT, kBK, kStages, kF32, kIT, kDual>), grid, dim3(128 * kWavesM), lds, s, p);
     return hipGetLastError();
 }
 
@@ -429,7 +548,7 @@ static int device_compute_units() {
 
 // Tile choice: time ~ (rounds of workgroups over the compute units) x (work per workgroup) / (efficiency of the tile);
 // larger tiles are more efficient (less L2 -> LDS traffic per flop) but leave compute units idle on small outputs.
-static int choose_tile(const GemmParams &p) {
+static int choose_tile(const GemmParams &p, double *model_time = nullptr) {
     static const int forced = getenv("RLLAMA_HIP_GEMM_TILE") ? atoi(getenv("RLLAMA_HIP_GEMM_TILE")) : -1;
     if (forced >= 1 && forced <= 3) return forced;
     const int k_halves = p.k * (p.f32_operands ? 2 : 1);
@@ -455,8 +574,9 @@ static int choose_tile(const GemmParams &p) {
         const long blocks = (long)((p.n + 63) / 64) * ((p.m + 127) / 128);
         const long rounds = (blocks + n_cu - 1) / n_cu;
         const double time = (double)rounds * 128 * 64 / 0.93;
-        if (time < best_t) best = 5;
+        if (time < best_t) { best = 5; best_t = time; }
     }
+    if (model_time != nullptr) *model_time = best_t;
     return best;
 }
 
@@ -486,7 +606,7 @@ __global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const float g = (float)g4[e];
-                o[e] = (half_t)(silu_fast(g) * f16r(acc[e]));
+                o[e] = to_f16(silu_fast(g) * f16r(acc[e]));
             }
             *reinterpret_cast<half4_t *>(reinterpret_cast<half_t *>(p.c) + off) = o;
         } else {
@@ -538,7 +658,7 @@ __global__ __launch_bounds__(256) void gemm_split_finish_norm_kernel(GemmParams 
             typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
             half4_t o;
 #pragma unroll
-            for (int e = 0; e < 4; e++) o[e] = (half_t)((xv[j][e] * rs) * wv[e]);
+            for (int e = 0; e < 4; e++) o[e] = to_f16((xv[j][e] * rs) * wv[e]);
             *reinterpret_cast<half4_t *>(yr + i * 4) = o;
         }
     }
@@ -578,9 +698,33 @@ static hipError_t launch_split_finish(const GemmParams &p, int splits, hipStream
     return hipGetLastError();
 }
 
+// Two products in one pass pay off where their workgroups (256 x 192 of both products each) fill the compute units about as
+// well as the best single-product tile does; shorter prompts keep the narrower tiles and split products of two launches.
+bool gemm_f16_dual_gate_supported(const GemmParams &p) {
+    const char *env = getenv("RLLAMA_HIP_GEMM_DUAL"); // 0: never, 1: wherever the kernel can run (tests), unset: by shape; read at every call
+    const int mode = env != nullptr ? atoi(env) : -1;
+    if (mode == 0 || p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.k % 64 != 0) return false;
+    if ((p.ldc % 8) != 0 || (p.n % 8) != 0 || (reinterpret_cast<uintptr_t>(p.c) % 16) != 0) return false;
+    if (mode == 1) return true;
+    // the tile model of choose_tile: two launches of the best single tile against the rounds of 256 x 192 workgroups that do
+    // both products, whose busy compute unit measured 1.18 of the single 256 x 192 tile's throughput (7B and 13B shapes, 256 to
+    // 2048 prompt rows: faster from 768 rows on except where the last round is nearly empty, slower at 256)
+    double single = 0.0;
+    const int tile = choose_tile(p, &single);
+    if (tile < 0 || tile > 3 || choose_split_k(p, tile) != 1) return false;
+    const int n_cu = device_compute_units();
+    const long blocks = (long)((p.n + 191) / 192) * ((p.m + 255) / 256);
+    const double dual = (double)((blocks + n_cu - 1) / n_cu) * 2.0 * 256 * 192 / (1.23 * 1.18);
+    return dual < 2.0 * single;
+}
+
 hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t s) {
     if (!gemm_f16_dma_supported(p_in) || p_in.m <= 0 || p_in.n <= 0 || p_in.batch < 1) return hipErrorInvalidValue;
     if (epilogue == kGemmEpiResAddF32 && (p_in.residual == nullptr || p_in.batch != 1)) return hipErrorInvalidValue;
+    if (p_in.b2 != nullptr) {
+        if (epilogue != kGemmEpiSiluGateF16 || !gemm_f16_dual_gate_supported(p_in)) return hipErrorInvalidValue;
+        return launch_dma<kGemmEpiSiluGateF16, 4, 3, 64, 2, false, 2, true>(p_in, s); // 256 x 192 of both products, all of the LDS
+    }
     if (epilogue == kGemmEpiSiluGateF16 && (p_in.gate == nullptr || p_in.batch != 1 || p_in.f32_operands)) return hipErrorInvalidValue;
     const int splits = choose_split_k(p_in, choose_tile(p_in));
     if (splits > 1) {

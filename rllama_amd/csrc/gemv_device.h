@@ -276,7 +276,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
             const int i = tid + j * kGemvThreads;
             if (i < n4) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) xs[i * 4 + e] = (XT)((xv[j][e] * rs) * wv[j][e]);
+                for (int e = 0; e < 4; e++) xs[i * 4 + e] = (XT)as_f32((xv[j][e] * rs) * wv[j][e]);
             }
         }
     } else if (p.norm_w != nullptr) {
@@ -294,7 +294,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
         for (int i = tid; i < K; i += kGemvThreads) {
             float v = act_load1<kDevLoad>(p.x + i);
             if (p.x_add != nullptr) v = v + act_load1<kDevLoad>(p.x_add + i);
-            xs[i] = (XT)((v * rs) * p.norm_w[i]);
+            xs[i] = (XT)as_f32((v * rs) * p.norm_w[i]);
         }
     } else {
         for (int base = 0; base < n4; base += kGemvPrologueVecs * kGemvThreads) {

@@ -113,6 +113,8 @@ struct GemmParams {
     void *c;                // [m x n], row stride ldc
     const float *residual;  // kGemmEpiResAddF32: [m x n], row stride ldc
     const _Float16 *gate;   // kGemmEpiSiluGateF16: [m x n], row stride ldc
+    const _Float16 *b2;     // kGemmEpiSiluGateF16, fast path, instead of gate: a second [n x k] matrix (row stride ldb); the gate is
+                            // f16(a * b^T), computed in the same pass, and C = SiLU(gate) * f16(a * b2^T) (gemm_f16_dual_gate_supported)
     int m, n, k;
     int lda, ldb, ldc;
     int batch;              // grid.z; element strides between batch items:
@@ -143,6 +145,8 @@ hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s);
 // fast path (gemm_dma.hip): k % 32 == 0; launch_gemm_f16 picks it when it applies
 bool gemm_f16_dma_supported(const GemmParams &p);
 hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s);
+// whether the fast path runs w1 and w3 of a feed-forward block (b, b2: both [n x k]) as one pass over A for this shape
+bool gemm_f16_dual_gate_supported(const GemmParams &p);
 
 // ---- prefill: element-wise kernels around the GEMMs (prefill.hip) ----
 struct PrefillRopeParams {

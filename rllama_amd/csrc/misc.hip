@@ -361,7 +361,7 @@ __global__ void silu_mul_f16_kernel(const half_t *g, const half_t *u, half_t *m,
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
         const float x = (float)g[i];
-        m[i] = (half_t)((x / (1.0f + expf(-x))) * (float)u[i]);
+        m[i] = to_f16((x / (1.0f + expf(-x))) * (float)u[i]);
     }
 }
 

@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_f16_kernel(half_t *y, const 
                 typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
                 half4_t o;
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (half_t)((xv[j][e] * rs) * wv[e]);
+                for (int e = 0; e < 4; e++) o[e] = to_f16((xv[j][e] * rs) * wv[e]);
                 *reinterpret_cast<half4_t *>(yr + i * 4) = o;
             }
         }
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_f16_kernel(half_t *y, const 
     for (int i = tid; i < d; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
     ss = block_sum(ss, red);
     const float rs = 1.0f / sqrtf(ss / (float)d + eps);
-    for (int i = tid; i < d; i += blockDim.x) yr[i] = (half_t)((xr[i] * rs) * w[i]);
+    for (int i = tid; i < d; i += blockDim.x) yr[i] = to_f16((xr[i] * rs) * w[i]);
 }
 
 hipError_t launch_rmsnorm_rows_f16(void *y, const float *x, const float *w, int rows, int d, float eps, hipStream_t s) {

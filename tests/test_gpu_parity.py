@@ -308,6 +308,31 @@ def test_prefill_wide_ffn_largest_tile(ctx):
     gm.free()
 
 
+@pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 1000, 300), (128, 2, 192, 256), (192, 3, 1544, 515)])
+def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n):
+    """w1 and w3 as one pass over the normalised rows (two accumulator sets per wavefront, SiLU(w1 x) * (w3 x) straight from
+    them: transformer.rs:551-565), forced onto shapes the oracle handles quickly: ragged last row and column tiles (300 and
+    515 rows on 256-row tiles, 1000 = 5 x 192 + 40 and 1544 = 8 x 192 + 8 columns), exactly one tile, three K-tiles.  Same
+    MFMA sequence per output element as the two-launch form, so the same bits; and against the oracle."""
+    shape = Shape(dim=dim, n_layers=2, n_heads=heads, ffn_hidden=ffn, vocab_size=64, max_seq_len=n + 2)
+    W = synth_weights(shape, seed=61, std=0.05, norm_ones=False)
+    toks = np.random.default_rng(62).integers(0, shape.vocab_size, n + 1)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    got = {}
+    for mode in ("1", "0"):
+        os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
+        try:
+            gc = gm.make_caches()
+            got[mode] = (gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc))
+        finally:
+            del os.environ["RLLAMA_HIP_GEMM_DUAL"]
+    assert np.array_equal(got["1"][0], got["0"][0]) and np.array_equal(got["1"][1], got["0"][1])
+    oc = om.make_caches()
+    assert max_rel_err(got["1"][0], om.forward(toks[:n], 0, oc)) < TOL_F16
+    assert max_rel_err(got["1"][1], om.forward(toks[n:n + 1], n, oc)) < TOL_F16
+    gm.free()
+
+
 def test_prefill_long_prompt_causal_tiles(ctx):
     """A prompt long enough that the score matrix spans several GEMM tiles per head (tiles above the diagonal are
     skipped, the probability product stops at the diagonal) on the large-tile path; compared with the oracle."""
