@@ -244,8 +244,13 @@ int  rlh_rope_inplace(rlh_tensor *x, int n_heads, int head_dim, int pos);
 /* Tensor::add (src/tensor.rs:573-593) as the residual adds use it (src/transformer.rs:442, 445): dst = a + b, f32. */
 int  rlh_add(rlh_tensor *dst, const rlh_tensor *a, const rlh_tensor *b);
 /* FeedForward's gate (src/transformer.rs:557-565): dst = silu(gate) * up, formed in f32 (src/tensor.rs:822-832, 722-734);
- * f16 tensors are read as f16 and the product is rounded to f16 once. */
+ * f16 tensors are read as f16, and the f32 product is rounded to f16 (the one rounding point). */
 int  rlh_silu_mul(rlh_tensor *dst, const rlh_tensor *gate, const rlh_tensor *up);
+/* FeedForward up to its gate for several rows at once, f16 mode (src/transformer.rs:551-565 with seq_len > 1):
+ * dst = f16(silu(f16(x * w1^T)) * f16(x * w3^T)); x [n x k], w1 and w3 [m x k], dst [n x m], all f16, k a multiple of 8.
+ * Where the shape fills the part, both products run as one matrix-core pass over x with two accumulator sets and the gate
+ * never reaches memory; otherwise as two products, the second consuming the first (same bits either way). */
+int  rlh_ffn_gate(rlh_tensor *dst, const rlh_tensor *x, const rlh_tensor *w1, const rlh_tensor *w3);
 /* One token's cache update (src/transformer.rs:704-761 with seq_len 1): RoPE on q (in place) and on k at position pos,
  * then k and v into the cache planes at pos (rounded to f16 for f16 planes).  q, k, v: f32, n_heads * head_dim elements. */
 int  rlh_rope_kvwrite(rlh_tensor *q, const rlh_tensor *k, const rlh_tensor *v, rlh_tensor *cache_k, rlh_tensor *cache_v, int n_heads,

@@ -383,6 +383,12 @@ class Tensor:
         check(self._lib.rlh_silu_mul(out._h, self._h, up._h))
         return out
 
+    def ffn_gate(self, w1: "Tensor", w3: "Tensor") -> "Tensor":
+        """self = x [n x k] f16: f16(silu(f16(x w1^T)) * f16(x w3^T)) for all rows at once (src/transformer.rs:551-565)."""
+        out = Tensor.zeros(self.ctx, self._rows, w1._rows, TensorDType.Float16)
+        check(self._lib.rlh_ffn_gate(out._h, self._h, w1._h, w3._h))
+        return out
+
     def rope_kvwrite(self, k: "Tensor", v: "Tensor", cache_k: "Tensor", cache_v: "Tensor", n_heads: int, max_seq_len: int, pos: int) -> None:
         """self = q: RoPE on q (in place) and k at pos; k and v into the cache planes at pos (src/transformer.rs:704-761)."""
         check(self._lib.rlh_rope_kvwrite(self._h, k._h, v._h, cache_k._h, cache_v._h, n_heads, max_seq_len, pos))

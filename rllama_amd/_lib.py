@@ -88,6 +88,7 @@ SIGNATURES = {
     "rlh_rope_inplace": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int]),
     "rlh_add": (C.c_int, [_vp, _vp, _vp]),
     "rlh_silu_mul": (C.c_int, [_vp, _vp, _vp]),
+    "rlh_ffn_gate": (C.c_int, [_vp, _vp, _vp, _vp]),
     "rlh_rope_kvwrite": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int]),
     "rlh_attn_decode": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "rlh_attn_decode_noalloc": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),

@@ -65,7 +65,7 @@ struct Layer {
 // Work buffers of a multi-token forward (prefill); grown on demand, kept for the next call.
 struct PrefillScratch {
     int n_cap = 0;       // rows the buffers are sized for
-    int t_pad = 0;       // n_cap rounded up to 64: row stride of scores / probabilities / transposed V
+    int t_pad = 0;       // n_cap rounded up to 128: row stride of scores / probabilities / transposed V
     float *x = nullptr, *h = nullptr, *scores = nullptr;
     // q2: rows [q hi | q lo] of 2 head_dim halves; p2: rows [P hi | P lo] of 2 t_pad halves (one GEMM sums both parts)
     void *xn = nullptr, *qkv = nullptr, *q2 = nullptr, *v_t = nullptr, *p2 = nullptr, *a = nullptr;
@@ -120,7 +120,10 @@ struct rlh_model {
     int prefill_mode = 0; // 0: matrix-core prefill where available (f16 mode), 1: token by token
     // fused attention kernel for multi-token calls (head_dim 64 / 128); RLLAMA_HIP_PREFILL_ATTN=gemm keeps the two-GEMM path
     bool prefill_attn_fused = !(getenv("RLLAMA_HIP_PREFILL_ATTN") && !strcmp(getenv("RLLAMA_HIP_PREFILL_ATTN"), "gemm"));
-    int prefill_attn_order = getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER") ? atoi(getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER")) : 2;
+    int prefill_attn_parts = getenv("RLLAMA_HIP_PREFILL_ATTN_PARTS") && atoi(getenv("RLLAMA_HIP_PREFILL_ATTN_PARTS")) == 4 ? 4 : 2;
+    // with two workgroups per compute unit (the four-wavefront form, the default) the second half of the grid runs upwards from
+    // the lightest query block; with one (the eight-wavefront form) the heaviest blocks go first
+    int prefill_attn_order = getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER") ? atoi(getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER")) : (prefill_attn_parts == 2 ? 2 : 1);
     // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
     uint64_t uid = 0;   // unique per created model: a later model at the same address is still another model
     int next_pos = -1;
@@ -878,7 +881,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     if (n <= S.n_cap) return RLH_OK;
     S.release();
     const size_t d = (size_t)m->prm.dim, F = (size_t)m->prm.ffn_hidden, H = (size_t)m->prm.n_heads, hd = (size_t)m->head_dim;
-    const size_t N = (size_t)n, tp = (N + 63) & ~(size_t)63;
+    const size_t N = (size_t)n, tp = (N + 127) & ~(size_t)127;
     const size_t es = m->prm.force_f16 ? 2 : 4; // element size of the activations between the GEMMs
     hipError_t e = hipSuccess;
     auto A = [&](void **p, size_t bytes) {
@@ -922,7 +925,7 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     const rlh_model_params &P = m->prm;
     PrefillScratch &S = m->pf;
     const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size, H = P.n_heads, hd = m->head_dim;
-    const int tp = (n + 63) & ~63; // row stride of this call's scores / probabilities / transposed V (a whole number of K-tiles)
+    const int tp = (n + 127) & ~127; // row stride of this call's scores / probabilities / transposed V (a whole number of key tiles)
     const float eps = (float)P.norm_eps;
     if (span) {
         HIP_TRY(hipMemcpyAsync(S.x, span->x_in, sizeof(float) * (size_t)n * d, hipMemcpyHostToDevice, st));
@@ -998,6 +1001,7 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
             ap.t_pad = tp;
             ap.scale = 1.0f / sqrtf((float)hd);
             ap.order = m->prefill_attn_order;
+            ap.key_parts = m->prefill_attn_parts;
             HIP_TRY(launch_attn_prefill(ap, st));
         } else {
             // scores[h] = q[h] . K[h]^T summed over the hi and lo parts of q: one pass that skips the tiles above the

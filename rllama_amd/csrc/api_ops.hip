@@ -276,6 +276,40 @@ extern "C" int rlh_silu_mul(rlh_tensor *dst, const rlh_tensor *gate, const rlh_t
     return RLH_OK;
 }
 
+extern "C" int rlh_ffn_gate(rlh_tensor *dst, const rlh_tensor *x, const rlh_tensor *w1, const rlh_tensor *w3) {
+    if (!dst || !x || !w1 || !w3) return fail(RLH_ERR_INVALID, "rlh_ffn_gate: NULL argument");
+    if (dst->dtype != RLH_F16 || x->dtype != RLH_F16 || w1->dtype != RLH_F16 || w3->dtype != RLH_F16) return fail(RLH_ERR_UNSUPPORTED, "rlh_ffn_gate: f16 tensors only");
+    if (!same_shape(w1, w3) || w1->cols != x->cols || dst->rows != x->rows || dst->cols != w1->rows) {
+        return fail(RLH_ERR_INVALID, "rlh_ffn_gate: shapes do not fit (x %dx%d, w1 %dx%d, w3 %dx%d, dst %dx%d)", x->rows, x->cols, w1->rows, w1->cols, w3->rows, w3->cols,
+                    dst->rows, dst->cols);
+    }
+    if (x->cols % 8 != 0) return fail(RLH_ERR_UNSUPPORTED, "rlh_ffn_gate: k must be a multiple of 8");
+    CtxLock lock(dst->ctx);
+    hipStream_t st = dst->ctx->stream;
+    GemmParams g{};
+    g.a = (const _Float16 *)x->p;
+    g.b = (const _Float16 *)w1->p;
+    g.c = dst->p;
+    g.m = x->rows;
+    g.n = w1->rows;
+    g.k = x->cols;
+    g.lda = g.ldb = x->cols;
+    g.ldc = w1->rows;
+    g.batch = 1;
+    GemmParams both = g;
+    both.b2 = (const _Float16 *)w3->p;
+    if (gemm_f16_dual_gate_supported(both)) { // both products in one pass over x
+        HIP_TRY(launch_gemm_f16(both, kGemmEpiSiluGateF16, st));
+        return RLH_OK;
+    }
+    // w1's product into dst, then w3's with dst as its gate: every element of the gate is read by the lane that overwrites it
+    HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
+    g.b = (const _Float16 *)w3->p;
+    g.gate = (const _Float16 *)dst->p;
+    HIP_TRY(launch_gemm_f16(g, kGemmEpiSiluGateF16, st));
+    return RLH_OK;
+}
+
 // (cos, sin) of compute_freqs_cis (transformer.rs:858-885) for positions first .. first + n - 1, as f32 like :836-837
 static std::vector<float2> rope_table(int head_dim, int first, int n) {
     std::vector<float2> tab((size_t)n * (head_dim / 2));
@@ -442,7 +476,7 @@ extern "C" int rlh_attn_prefill(rlh_tensor *out, const rlh_tensor *qkv, rlh_tens
     rlh_ctx *ctx = out->ctx;
     CtxLock lock(ctx);
     hipStream_t st = ctx->stream;
-    const int tp = (n + 63) & ~63;
+    const int tp = (n + 127) & ~127;
     const std::vector<float2> tab = rope_table(hd, 0, n);
     float2 *freqs = nullptr;
     void *q2 = nullptr, *v_t = nullptr;
@@ -484,7 +518,9 @@ extern "C" int rlh_attn_prefill(rlh_tensor *out, const rlh_tensor *qkv, rlh_tens
         ap.max_seq_len = max_seq_len;
         ap.t_pad = tp;
         ap.scale = 1.0f / sqrtf((float)hd);
-        ap.order = 2;
+        const char *parts = getenv("RLLAMA_HIP_PREFILL_ATTN_PARTS"); // 4: the eight-wavefront form (read at every call)
+        ap.key_parts = parts != nullptr && atoi(parts) == 4 ? 4 : 2;
+        ap.order = ap.key_parts == 2 ? 2 : 1;
         e = launch_attn_prefill(ap, st);
     }
     hipError_t e2 = hipStreamSynchronize(st);

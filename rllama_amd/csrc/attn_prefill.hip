@@ -8,13 +8,14 @@
 // rescaled accumulator; exponentials through exp2), which is the same function as exp(s) / sum exp(s) wherever that is
 // finite.  The output is rounded to f16 where the reference does (transformer.rs:793-796).
 //
-// Blocking.  Workgroup = 4 wavefronts = 64 queries of one head.  Wavefront (g, h) owns the 32 queries of query group g
-// and, of every 64-key tile, the 32 keys of key half h; the two halves keep their own (m, l, O) and are merged through
-// LDS at the end.  Splitting the keys rather than taking more queries doubles the number of workgroups (two fit on a
-// compute unit, so every SIMD holds two wavefronts and one's softmax arithmetic overlaps the other's MFMAs) and lets
-// light and heavy query blocks (1 .. n / 64 key tiles, causal) share a compute unit.  The K tile [64 x hd] and the V^T
-// tile [hd x 64] go from global memory straight into LDS (global_load_lds, two stages: the next tile's loads are in
-// flight while the current one is used; one barrier per tile).
+// Blocking.  Workgroup = 2 KQ wavefronts = 64 queries of one head.  Wavefront (g, h) owns the 32 queries of query group g
+// and, of every key tile of 32 KQ keys, the 32 keys of key part h; the parts keep their own (m, l, O) and are merged
+// through LDS at the end.  Splitting the keys rather than taking more queries gives every SIMD two wavefronts, so that
+// one's softmax arithmetic overlaps the other's MFMAs.  KQ = 2 (four wavefronts, 64-key tiles, two workgroups per compute
+// unit) is what runs; KQ = 4 (eight wavefronts, 128-key tiles, one workgroup per compute unit, which keeps two wavefronts
+// on every SIMD for the whole life of a heavy query block) measured 1 % slower on whole 7B prompts of 1024 and 2048 tokens
+// and is kept as the comparison.  The K tile [keys x hd] and the V^T tile [hd x keys] go from global memory straight into LDS
+// (global_load_lds, two stages: the next tile's loads are in flight while the current one is used; one barrier per tile).
 //
 // Both products are computed transposed so that every per-query quantity lives in one lane pair:
 //   S^T [key x query]  = K (A operand, rows = keys)   x  q (B operand, rows = queries), summed over hd
@@ -35,32 +36,33 @@ typedef __attribute__((ext_vector_type(16))) float float16_t;
 typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
 
 constexpr int kApQueries = 64; // per workgroup
-constexpr int kApKeys = 64;    // per key tile
-constexpr int kApThreads = 256;
 
-template <int HD>
-__global__ __launch_bounds__(kApThreads, 2) void attn_prefill_kernel(AttnPrefillParams p) {
+template <int HD, int KQ>
+__global__ __launch_bounds__(128 * KQ, KQ == 2 ? 2 : 1) void attn_prefill_kernel(AttnPrefillParams p) {
+    constexpr int kApKeys = 32 * KQ;              // per key tile
+    constexpr int kWaves = 2 * KQ;
     constexpr int kKS = HD / 16;                  // MFMA K-steps over the head dimension
     constexpr int kDT = HD / 32;                  // 32-row tiles of O^T
     constexpr int kKRowBytes = HD * 2;            // K tile row (one key)
     constexpr int kKChunks = HD / 8;              // 16-byte chunks per K row
     constexpr int kKSwzDiv = 16 / kKChunks;       // K rows per 256 bytes of LDS: rows that start in the same bank
     constexpr int kKTileBytes = kApKeys * kKRowBytes;
-    constexpr int kVRowBytes = kApKeys * 2;       // V^T tile row (one dim): 128 bytes = 8 chunks
+    constexpr int kVRowBytes = kApKeys * 2;       // V^T tile row (one dim): 8 or 16 chunks
+    constexpr int kVChunks = kApKeys / 8;
     constexpr int kVTileBytes = HD * kVRowBytes;
     constexpr int kStageBytes = kKTileBytes + kVTileBytes;
-    constexpr int kKIssues = kKTileBytes / 4096;  // wavefront-wide 1 KiB loads per wavefront and tile
-    constexpr int kVIssues = kVTileBytes / 4096;
-    constexpr int kMergeFloats = 64 * (kDT * 16 + 2); // one key half's (O, m, l), a float per lane and value
+    constexpr int kKIssues = kKTileBytes / (kWaves * 1024);  // wavefront-wide 1 KiB loads per wavefront and tile
+    constexpr int kVIssues = kVTileBytes / (kWaves * 1024);
+    constexpr int kMergeFloats = 64 * (kDT * 16 + 2); // one key part's (O, m, l), a float per lane and value
     constexpr int kOutRowHalves = HD + 8;         // padded row of the f16 output tile
-    constexpr int kOutOffset = 2 * kMergeFloats * 4;
+    constexpr int kOutOffset = 2 * (KQ - 1) * kMergeFloats * 4;
     static_assert(kOutOffset + 2 * 32 * kOutRowHalves * 2 <= 2 * kStageBytes, "epilogue buffers reuse the tile stages");
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int qg = wave & 1, kh = wave >> 1;
+    const int qg = wave & 1, kh = wave >> 1;      // query group, key part
     const int col = lane & 31, half = lane >> 5;
     const int n = p.n;
     const int n_qblocks = (n + kApQueries - 1) / kApQueries;
@@ -105,36 +107,37 @@ __global__ __launch_bounds__(kApThreads, 2) void attn_prefill_kernel(AttnPrefill
         for (int v = 0; v < 16; v++) o_acc[d][v] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;
 
-    // keys 0 .. qblock + 63 matter to this workgroup (causal), i.e. key tiles 0 .. qi
-    const int n_tiles = qi + 1;
+    // keys 0 .. qblock + 63 matter to this workgroup (causal)
+    const int n_tiles = (qblock + kApQueries + kApKeys - 1) / kApKeys;
 
     // ---- staging.  Load i of wavefront w fills LDS bytes (4 i + w) * 1024 .. + 1024 of the tile; lane l's 16 bytes are
     //      chunk position l % chunks of row l / chunks, which holds the row's chunk (position ^ f(row)): consecutive
     //      rows put the same logical chunk into different banks, which makes the MFMA operand reads conflict-free.
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds;
+    auto v_swz = [](int row) { return kVChunks == 8 ? (row >> 1) & 7 : row & 15; }; // 16 consecutive rows of V^T: 16 distinct 16-byte bank groups
     int k_row[kKIssues], k_off[kKIssues], v_off[kVIssues];
 #pragma unroll
     for (int i = 0; i < kKIssues; i++) {
-        const int L = (i * 4 + wave) * 64 + lane;
+        const int L = (i * kWaves + wave) * 64 + lane;
         const int row = L / kKChunks, cp = L % kKChunks;
         k_row[i] = row;
         k_off[i] = (cp ^ ((row / kKSwzDiv) & (kKChunks - 1))) * 8;
     }
 #pragma unroll
     for (int i = 0; i < kVIssues; i++) {
-        const int L = (i * 4 + wave) * 64 + lane;
-        const int row = L / 8, cp = L % 8;
-        v_off[i] = row * p.t_pad + (cp ^ ((row >> 1) & 7)) * 8;
+        const int L = (i * kWaves + wave) * 64 + lane;
+        const int row = L / kVChunks, cp = L % kVChunks;
+        v_off[i] = row * p.t_pad + (cp ^ v_swz(row)) * 8;
     }
     auto issue = [&](int kt) {
         const unsigned dst = lds_base + (unsigned)(kt & 1) * kStageBytes + (unsigned)wave * 1024;
 #pragma unroll
         for (int i = 0; i < kKIssues; i++) {
             const int key = min(kt * kApKeys + k_row[i], p.max_seq_len - 1); // keys past the sequence are masked below
-            dma16(kbase + (size_t)key * HD + k_off[i], dst + i * 4096);
+            dma16(kbase + (size_t)key * HD + k_off[i], dst + i * (kWaves * 1024));
         }
 #pragma unroll
-        for (int i = 0; i < kVIssues; i++) dma16(vbase + (size_t)(kt * kApKeys) + v_off[i], dst + kKTileBytes + i * 4096);
+        for (int i = 0; i < kVIssues; i++) dma16(vbase + (size_t)(kt * kApKeys) + v_off[i], dst + kKTileBytes + i * (kWaves * 1024));
     };
 
     const float c2 = p.scale * 1.44269504088896340736f;
@@ -219,33 +222,43 @@ __global__ __launch_bounds__(kApThreads, 2) void attn_prefill_kernel(AttnPrefill
 #pragma unroll
             for (int d = 0; d < kDT; d++) {
                 const int vrow = d * 32 + col;
-                const half8_t vf = *reinterpret_cast<const half8_t *>(lds_v + vrow * kVRowBytes + ((ch ^ ((vrow >> 1) & 7)) << 4));
+                const half8_t vf = *reinterpret_cast<const half8_t *>(lds_v + vrow * kVRowBytes + ((ch ^ v_swz(vrow)) << 4));
                 o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, p_hi, o_acc[d], 0, 0, 0);
                 o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, p_lo, o_acc[d], 0, 0, 0);
             }
         }
     }
 
-    // ---- merge the two key halves: wavefront (g, 1) hands (O, m, l) to wavefront (g, 0) through LDS
+    // ---- merge the key parts: wavefronts (g, 1 ..) hand (O, m, l) to wavefront (g, 0) through LDS
     __syncthreads(); // every wavefront is done with the tiles (all loads were waited for above)
-    float *mb = reinterpret_cast<float *>(lds) + qg * kMergeFloats + lane;
-    if (kh == 1) {
+    float *mb = reinterpret_cast<float *>(lds) + qg * ((KQ - 1) * kMergeFloats) + lane;
+    if (kh > 0) {
+        float *mine = mb + (kh - 1) * kMergeFloats;
 #pragma unroll
         for (int d = 0; d < kDT; d++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) mb[(d * 16 + v) * 64] = o_acc[d][v];
-        mb[(kDT * 16) * 64] = m_run;
-        mb[(kDT * 16 + 1) * 64] = l_run;
+            for (int v = 0; v < 16; v++) mine[(d * 16 + v) * 64] = o_acc[d][v];
+        mine[(kDT * 16) * 64] = m_run;
+        mine[(kDT * 16 + 1) * 64] = l_run;
     }
     __syncthreads();
-    if (kh == 1) return;
+    if (kh > 0) return;
     {
-        const float m1 = mb[(kDT * 16) * 64], l1 = mb[(kDT * 16 + 1) * 64];
-        const float m = fmaxf(m_run, m1); // m_run is finite (key 0 <= every query); m1 is -inf if the half saw no key
-        const float a0 = __builtin_amdgcn_exp2f((m_run - m) * c2), a1 = __builtin_amdgcn_exp2f((m1 - m) * c2);
-        const float l_half = l_run * a0 + l1 * a1;
+        // m_run is finite (key 0 <= every query); another part's maximum is -inf if it saw no key
+        float m = m_run;
+#pragma unroll
+        for (int j = 0; j < KQ - 1; j++) m = fmaxf(m, mb[j * kMergeFloats + (kDT * 16) * 64]);
+        float a[KQ];
+        a[0] = __builtin_amdgcn_exp2f((m_run - m) * c2);
+        float l_half = l_run * a[0];
+#pragma unroll
+        for (int j = 0; j < KQ - 1; j++) {
+            a[j + 1] = __builtin_amdgcn_exp2f((mb[j * kMergeFloats + (kDT * 16) * 64] - m) * c2);
+            l_half += mb[j * kMergeFloats + (kDT * 16 + 1) * 64] * a[j + 1];
+        }
         const float l_tot = l_half + __shfl_xor(l_half, 32, 64);
-        const float inv0 = a0 / l_tot, inv1 = a1 / l_tot;
+#pragma unroll
+        for (int j = 0; j < KQ; j++) a[j] = a[j] / l_tot;
         // normalise, round to f16 (transformer.rs:793-796) and turn O^T into rows of the output through LDS, so that
         // the stores to memory are whole 16-byte pieces of consecutive columns
         half_t *ot = reinterpret_cast<half_t *>(lds + kOutOffset) + qg * (32 * kOutRowHalves);
@@ -255,7 +268,12 @@ __global__ __launch_bounds__(kApThreads, 2) void attn_prefill_kernel(AttnPrefill
             for (int g = 0; g < 4; g++) {
                 half4_t o;
 #pragma unroll
-                for (int i = 0; i < 4; i++) o[i] = to_f16(o_acc[d][g * 4 + i] * inv0 + mb[(d * 16 + g * 4 + i) * 64] * inv1);
+                for (int i = 0; i < 4; i++) {
+                    float sum = o_acc[d][g * 4 + i] * a[0];
+#pragma unroll
+                    for (int j = 0; j < KQ - 1; j++) sum += mb[j * kMergeFloats + (d * 16 + g * 4 + i) * 64] * a[j + 1];
+                    o[i] = to_f16(sum);
+                }
                 *reinterpret_cast<half4_t *>(ot + col * kOutRowHalves + d * 32 + g * 8 + half * 4) = o;
             }
         // rows q0 .. q0 + 31, columns head * HD .. + HD of wo's input
@@ -273,13 +291,15 @@ __global__ __launch_bounds__(kApThreads, 2) void attn_prefill_kernel(AttnPrefill
 bool attn_prefill_supported(int head_dim) { return head_dim == 64 || head_dim == 128; }
 
 hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s) {
-    if (p.n < 1 || p.n_heads < 1 || (p.t_pad % kApKeys) != 0 || p.t_pad < p.n || (p.dim % 8) != 0 || p.max_seq_len < 1) return hipErrorInvalidValue;
+    // key tiles of 64 (four wavefronts) unless asked for the eight-wavefront form; t_pad covers whole key tiles either way
+    const bool four = p.key_parts != 4;
+    if (p.n < 1 || p.n_heads < 1 || (p.t_pad % (four ? 64 : 128)) != 0 || p.t_pad < p.n || (p.dim % 8) != 0 || p.max_seq_len < 1) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((p.n + kApQueries - 1) / kApQueries * p.n_heads));
-    switch (p.head_dim) {
-    case 64: hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, dim3(kApThreads), 0, s, p); break;
-    case 128: hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, dim3(kApThreads), 0, s, p); break;
-    default: return hipErrorInvalidValue;
-    }
+    if (p.head_dim == 64 && four) hipLaunchKernelGGL((attn_prefill_kernel<64, 2>), grid, dim3(256), 0, s, p);
+    else if (p.head_dim == 64) hipLaunchKernelGGL((attn_prefill_kernel<64, 4>), grid, dim3(512), 0, s, p);
+    else if (p.head_dim == 128 && four) hipLaunchKernelGGL((attn_prefill_kernel<128, 2>), grid, dim3(256), 0, s, p);
+    else if (p.head_dim == 128) hipLaunchKernelGGL((attn_prefill_kernel<128, 4>), grid, dim3(512), 0, s, p);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 

@@ -526,7 +526,10 @@ static hipError_t launch_dma_epi(const GemmParams &p, int tile, hipStream_t s) {
     const bool k64 = p.k % 64 == 0 && (p.k_seg == 0 || p.k_seg % 64 == 0);
     switch (tile) {
     case 0: return launch_dma<kEpi, 2, 2, 64, 2>(p, s);  // 128 x 128, 64 KiB of LDS: two workgroups per compute unit
-    case 4: return launch_dma<kEpi, 2, 2, 64, 4>(p, s);  // 128 x 128, 128 KiB: one workgroup per compute unit, three K-tiles ahead
+#ifndef RLH_T4_ARGS
+#define RLH_T4_ARGS 2, 2, 64, 4
+#endif
+    case 4: return launch_dma<kEpi, RLH_T4_ARGS>(p, s);  // 128 x 128, 128 KiB: one workgroup per compute unit, three K-tiles ahead
     case 5: return launch_dma<kEpi, 2, 1, 64, 6>(p, s);  // 128 x 64, 144 KiB: few rows, so twice the workgroups stream the weights
     case 6: return launch_dma<kEpi, 1, 1, 64, 10, false, 1>(p, s);  // 32 x 64, 120 KiB: at most 32 rows, nine weight tiles in flight per workgroup
     case 7: return launch_dma<kEpi, 1, 1, 64, 8, false, 2>(p, s);   // 64 x 64, 128 KiB: at most 64 rows

@@ -169,6 +169,7 @@ struct AttnPrefillParams {
     int n, n_heads, head_dim, dim, max_seq_len, t_pad;
     float scale;             // 1 / sqrt(head_dim) (transformer.rs:770)
     int order;               // launch order of the query blocks: 0 ascending, 1 descending, 2 descending then ascending
+    int key_parts;           // 2 (or 0): four wavefronts on 64-key tiles, t_pad % 64 == 0; 4: eight wavefronts on 128-key tiles, t_pad % 128 == 0
 };
 bool attn_prefill_supported(int head_dim);
 hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s);

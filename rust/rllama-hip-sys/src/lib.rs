@@ -127,6 +127,7 @@ extern "C" {
     pub fn rlh_rope_inplace(x: *mut rlh_tensor, n_heads: c_int, head_dim: c_int, pos: c_int) -> c_int;
     pub fn rlh_add(dst: *mut rlh_tensor, a: *const rlh_tensor, b: *const rlh_tensor) -> c_int;
     pub fn rlh_silu_mul(dst: *mut rlh_tensor, gate: *const rlh_tensor, up: *const rlh_tensor) -> c_int;
+    pub fn rlh_ffn_gate(dst: *mut rlh_tensor, x: *const rlh_tensor, w1: *const rlh_tensor, w3: *const rlh_tensor) -> c_int;
     pub fn rlh_rope_kvwrite(q: *mut rlh_tensor, k: *const rlh_tensor, v: *const rlh_tensor, cache_k: *mut rlh_tensor, cache_v: *mut rlh_tensor, n_heads: c_int, max_seq_len: c_int, pos: c_int) -> c_int;
     pub fn rlh_attn_decode(out: *mut rlh_tensor, q: *const rlh_tensor, cache_k: *const rlh_tensor, cache_v: *const rlh_tensor, n_heads: c_int, max_seq_len: c_int, T: c_int, n_splits: c_int, round_out: c_int) -> c_int;
     pub fn rlh_attn_decode_noalloc(out: *mut rlh_tensor, q: *const rlh_tensor, cache_k: *const rlh_tensor, cache_v: *const rlh_tensor, n_heads: c_int, max_seq_len: c_int, T: c_int, n_splits: c_int, round_out: c_int) -> c_int;

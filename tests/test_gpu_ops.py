@@ -174,11 +174,47 @@ def test_add_and_silu_mul(ctx):
         Tensor.from_numpy(ctx, ah).add(Tensor.from_numpy(ctx, bh))                                   # the residual stream is f32
 
 
+@pytest.mark.parametrize("n,m,k", [(300, 1000, 256), (256, 192, 64), (70, 520, 128), (513, 392, 192)])
+def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
+    """FeedForward up to its gate for n rows (src/transformer.rs:551-565): the oracle's f16 matmul (src/tensor.rs:1282-1475,
+    result rounded to f16), silu and hadamard product in f32, one rounding to f16.  The matrix cores add the k products in
+    another order than the reference's lanes, so a product near an f16 rounding boundary may land on the neighbouring value:
+    at most one f16 step, on few elements.  The one-pass form (forced) and the two-product form give the same bits."""
+    import os
+    rng = np.random.default_rng(n + m + k)
+    x = (rng.standard_normal((n, k)) * 0.5).astype(np.float16)
+    w1 = (rng.standard_normal((m, k)) * 0.1).astype(np.float16)
+    w3 = (rng.standard_normal((m, k)) * 0.1).astype(np.float16)
+    g = oracle.matmul_transposed_f16(x.view(np.uint16), w1.view(np.uint16)).view(np.float16).astype(f32)
+    u = oracle.matmul_transposed_f16(x.view(np.uint16), w3.view(np.uint16)).view(np.float16).astype(f32)
+    silu = np.array([oracle.silu(float(v)) for v in g.ravel()], f32).reshape(g.shape)
+    want = (silu * u).astype(np.float16)
+    X, W1, W3 = Tensor.from_numpy(ctx, x), Tensor.from_numpy(ctx, w1), Tensor.from_numpy(ctx, w3)
+    got = {}
+    for mode in ("1", "0"):
+        os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
+        try:
+            got[mode] = X.ffn_gate(W1, W3).to_numpy()
+        finally:
+            del os.environ["RLLAMA_HIP_GEMM_DUAL"]
+    assert np.array_equal(got["1"].view(np.uint16), got["0"].view(np.uint16))
+    one = got["1"]
+    step = np.spacing(np.maximum(np.abs(want), np.abs(one))).astype(f32)
+    assert np.mean(one != want) < 2e-2 and np.all(np.abs(one.astype(f32) - want.astype(f32)) <= 2 * step)
+    with pytest.raises(rllama_amd.RllamaHipError):
+        X.ffn_gate(W1, Tensor.from_numpy(ctx, w3[:-1]))                                              # w1 and w3 of two shapes
+    with pytest.raises(rllama_amd.RllamaHipError):
+        Tensor.from_numpy(ctx, x.astype(f32)).ffn_gate(W1, W3)                                       # f16 mode only
+
+
+@pytest.mark.parametrize("parts", [2, 4])
 @pytest.mark.parametrize("hd,H,n", [(128, 2, 200), (64, 3, 65), (128, 1, 64), (64, 2, 1), (128, 2, 333)])
-def test_attn_prefill_against_the_reference_ops(ctx, hd, H, n):
+def test_attn_prefill_against_the_reference_ops(ctx, hd, H, n, parts, monkeypatch):
     """The prompt's attention block between the projections and wo against the oracle's restatement of
     src/transformer.rs:704-796: RoPE, f16 cache rows, per row scores by the sequential-k product (src/tensor.rs:1050-1115),
-    mask, softmax, P.V by dot8, heads concatenated and rounded to f16.  Ragged query / key tiles included."""
+    mask, softmax, P.V by dot8, heads concatenated and rounded to f16.  Ragged query / key tiles included; both forms of the
+    kernel (four wavefronts on 64-key tiles, eight on 128-key tiles)."""
+    monkeypatch.setenv("RLLAMA_HIP_PREFILL_ATTN_PARTS", str(parts))
     rng = np.random.default_rng(hd + H * 13 + n)
     d, S = H * hd, 352
     qkv = (rng.standard_normal((n, 3 * d)) * 0.8).astype(np.float16)
