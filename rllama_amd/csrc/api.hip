@@ -967,7 +967,6 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         char *ck = (char *)c->k + (size_t)l * layer_elems * 2;
         char *cv = (char *)c->v + (size_t)l * layer_elems * 2;
         if (!normed) HIP_TRY(launch_rmsnorm_rows_f16(S.xn, S.x, (const float *)L.attn_norm.p, n, d, eps, st));
-        if ((rc = gemm(S.xn, d, L.wqkv.p, d, S.qkv, 3 * d, n, 3 * d, d, kGemmEpiF16, nullptr)) != RLH_OK) return rc;
         PrefillRopeParams rp{};
         rp.qkv = S.qkv;
         rp.freqs = m->freqs;
@@ -985,7 +984,29 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         rp.t_pad = tp;
         const bool fused = m->prefill_attn_fused && attn_prefill_supported(hd);
         rp.vt_swap = fused ? 1 : 0;
-        HIP_TRY(launch_rope_kv_prefill(rp, st));
+        {
+            // wq|wk|wv; RoPE, the hi + lo halves of q, the cache rows and V^T come straight out of the product's epilogue where
+            // the shape allows, else the product is stored and a kernel of its own does the same
+            GemmParams g{};
+            g.a = (const _Float16 *)S.xn;
+            g.b = (const _Float16 *)L.wqkv.p;
+            g.c = S.qkv;
+            g.m = n;
+            g.n = 3 * d;
+            g.k = d;
+            g.lda = g.ldb = d;
+            g.ldc = 3 * d;
+            g.batch = 1;
+            g.workspace = S.gemm_ws;
+            g.workspace_bytes = PrefillScratch::kGemmWsBytes;
+            g.rope = rp;
+            if (gemm_f16_rope_supported(g)) {
+                HIP_TRY(launch_gemm_f16(g, kGemmEpiRopeQkv, st));
+            } else {
+                HIP_TRY(launch_gemm_f16(g, kGemmEpiF16, st));
+                HIP_TRY(launch_rope_kv_prefill(rp, st));
+            }
+        }
         if (fused) {
             // scores, mask, softmax and P.V in one kernel; the score matrix never reaches memory
             AttnPrefillParams ap{};

@@ -135,6 +135,7 @@ hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s) {
         return launch_gemm_f16_dma(p, epilogue, s);
     }
     if (p.m <= 0 || p.n <= 0 || p.k <= 0 || (p.k % 8) != 0 || (p.lda % 8) != 0 || (p.ldb % 8) != 0 || p.batch < 1) return hipErrorInvalidValue;
+    if (epilogue == kGemmEpiRopeQkv) return gemm_f16_rope_supported(p) ? launch_gemm_f16_dma(p, epilogue, s) : hipErrorInvalidValue; // fast path only
     if (p.b2 != nullptr) return gemm_f16_dual_gate_supported(p) ? launch_gemm_f16_dma(p, epilogue, s) : hipErrorInvalidValue; // fast path only
     // RLLAMA_HIP_GEMM_SIMPLE=1 keeps every product on the kernel of this file (tuning / cross-checks)
     static const bool simple_only = getenv("RLLAMA_HIP_GEMM_SIMPLE") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_SIMPLE")) != 0;

@@ -380,6 +380,88 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
     // f16 outputs whose rows are 16-byte aligned go through LDS (the stages are free now): every wavefront lays its 64 x 32 kNT
     // tile out as rows, then stores whole 16-byte pieces of consecutive columns (and, with the SiLU gate, reads the gate the
     // same way) instead of one 2-byte element per lane and accumulator register.
+    if constexpr (kEpi == kGemmEpiRopeQkv) {
+        // The product of wq|wk|wv never reaches memory: every wavefront lays its f16-rounded tile (tensor.rs:1623-1643) out
+        // as rows in LDS and then handles it in 16-byte pieces of 8 consecutive columns, each of which lies within q, k or v
+        // of one head: RoPE on q and k in fp32 (transformer.rs:823-856), q as hi + lo f16 halves for the attention kernel, k
+        // and v rounded into the cache (tensor.rs:373-376), and v once more transposed, 8 positions per piece.
+        const PrefillRopeParams &R = p.rope;
+        constexpr int kTW = 32 * kNT;
+        constexpr int kPad = (kWaves * kWR * (kTW + 8) * 2 <= kStages * kStageBytes) ? 8 : 0;
+        constexpr int kTS = kTW + kPad;
+        static_assert(kWaves * kWR * kTS * 2 <= kStages * kStageBytes, "the output tiles reuse the stages");
+        constexpr int kChunks = kTW / 8;
+        __syncthreads(); // every wavefront has read its last fragments
+        half_t *tile = reinterpret_cast<half_t *>(lds_raw) + wave * (kWR * kTS);
+#pragma unroll
+        for (int i = 0; i < kIT; i++)
+#pragma unroll
+            for (int j = 0; j < kNT; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) tile[(i * 32 + (v >> 2) * 8 + row_in + (v & 3)) * kTS + j * 32 + col_in] = (half_t)acc[i][j][v];
+        const int d = R.dim, hd = R.head_dim, half_hd = hd / 2;
+        half_t *qhi = reinterpret_cast<half_t *>(R.q_hi), *qlo = reinterpret_cast<half_t *>(R.q_lo);
+        half_t *ck = reinterpret_cast<half_t *>(R.cache_k), *cv = reinterpret_cast<half_t *>(R.cache_v);
+        const int wr0 = bm0 + wm * kWR, wc0 = bn0 + wn * kTW; // first row (position) and column of this wavefront's tile
+#pragma unroll
+        for (int it = 0; it < kChunks * kWR / 64; it++) {
+            const int idx = it * 64 + lane;
+            const int rr = idx / kChunks, ch = idx - rr * kChunks;
+            const int r = wr0 + rr, c = wc0 + ch * 8;
+            if (r < M && c < N) {
+                const half8_t o = *reinterpret_cast<const half8_t *>(tile + rr * kTS + ch * 8);
+                const int part = c / d, cin = c - part * d; // 0 q, 1 k, 2 v
+                const int head = cin / hd, d0 = cin - head * hd;
+                const size_t co = ((size_t)head * R.max_seq_len + r) * hd + d0;
+                if (part == 2) {
+                    *reinterpret_cast<half8_t *>(cv + co) = o;
+                } else {
+                    const float2 *fr = R.freqs + (size_t)r * half_hd + d0 / 2;
+                    half8_t hi, lo;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        float a, b;
+                        rope_pair((float)o[2 * e], (float)o[2 * e + 1], fr[e], a, b);
+                        hi[2 * e] = (half_t)a;
+                        hi[2 * e + 1] = (half_t)b;
+                        lo[2 * e] = (half_t)(a - (float)hi[2 * e]);
+                        lo[2 * e + 1] = (half_t)(b - (float)hi[2 * e + 1]);
+                    }
+                    if (part == 0) {
+                        const size_t qo = ((size_t)head * M + r) * R.q_stride + d0;
+                        *reinterpret_cast<half8_t *>(qhi + qo) = hi;
+                        *reinterpret_cast<half8_t *>(qlo + qo) = lo;
+                    } else {
+                        *reinterpret_cast<half8_t *>(ck + co) = hi; // the rotated k rounded to f16
+                    }
+                }
+            }
+        }
+        // V^T [dim][t_pad]: 8 consecutive (stored) positions of one column per piece; eight lanes cover the 64 positions of a
+        // column, i.e. 128 contiguous bytes.  Rows past m hold copies of the last row (finite), which is what the padding of
+        // V^T needs.  With vt_swap the stored order within every 16 positions has bits 2 and 3 of the position exchanged.
+        if (wc0 + kTW > 2 * d) {
+            half_t *vt = reinterpret_cast<half_t *>(R.v_t);
+            constexpr int kPieces = kWR / 8;
+#pragma unroll
+            for (int it = 0; it < kTW * kPieces / 64; it++) {
+                const int idx = it * 64 + lane;
+                const int cc = idx / kPieces, j = idx - cc * kPieces;
+                const int c = wc0 + cc, pos0 = wr0 + j * 8;
+                if (c >= 2 * d && c < N && pos0 < R.t_pad) {
+                    half8_t o;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const int rs = j * 8 + e;
+                        const int src = R.vt_swap ? (rs & ~12) | ((rs & 4) << 1) | ((rs & 8) >> 1) : rs;
+                        o[e] = tile[src * kTS + cc];
+                    }
+                    *reinterpret_cast<half8_t *>(vt + (size_t)(c - 2 * d) * R.t_pad + pos0) = o;
+                }
+            }
+        }
+        return;
+    }
     if constexpr (kEpi == kGemmEpiF16 || kEpi == kGemmEpiSiluGateF16) {
         if (rows16) { // uniform for the launch
             constexpr int kTW = 32 * kNT; // tile width of a wavefront
@@ -471,6 +553,8 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                         reinterpret_cast<half_t *>(p.c)[off] = (half_t)val; // tensor.rs:1623-1643
                     } else if constexpr (kEpi == kGemmEpiF32) {
                         reinterpret_cast<float *>(p.c)[off] = prev[i][v] + val;
+                    } else if constexpr (kEpi == kGemmEpiRopeQkv) {
+                        (void)val; // returned above
                     } else if constexpr (kEpi == kGemmEpiSiluGateF16) { // tensor.rs:822-832 on the f16 gate, times the f16-rounded product
                         const float g = prev[i][v];
                         reinterpret_cast<half_t *>(p.c)[off] = to_f16(silu_fast(g) * f16r(val));
@@ -721,9 +805,25 @@ bool gemm_f16_dual_gate_supported(const GemmParams &p) {
     return dual < 2.0 * single;
 }
 
+// The RoPE epilogue needs whole 16-byte pieces everywhere and an unsplit product (a product cut along K has its epilogue in
+// the kernel that adds the partial sums; the caller then stores the product and runs the separate kernel).
+bool gemm_f16_rope_supported(const GemmParams &p) {
+    const char *env = getenv("RLLAMA_HIP_GEMM_ROPE"); // 0: never (the separate kernel); read at every call
+    if (env != nullptr && atoi(env) == 0) return false;
+    const PrefillRopeParams &R = p.rope;
+    if (p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.b2 != nullptr) return false;
+    if (R.dim <= 0 || R.head_dim <= 0 || p.n != 3 * R.dim || R.n != p.m || R.dim % R.head_dim != 0 || R.head_dim % 8 != 0 || !R.cache_f16) return false;
+    if (R.q_stride % 8 != 0 || R.t_pad % 8 != 0 || R.t_pad < p.m || p.m > R.max_seq_len) return false;
+    for (const void *q : {(const void *)R.q_hi, (const void *)R.q_lo, (const void *)R.cache_k, (const void *)R.cache_v, (const void *)R.v_t})
+        if (q == nullptr || (reinterpret_cast<uintptr_t>(q) % 16) != 0) return false;
+    if (R.freqs == nullptr || (reinterpret_cast<uintptr_t>(R.freqs) % 8) != 0) return false;
+    return choose_split_k(p, choose_tile(p)) == 1;
+}
+
 hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t s) {
     if (!gemm_f16_dma_supported(p_in) || p_in.m <= 0 || p_in.n <= 0 || p_in.batch < 1) return hipErrorInvalidValue;
     if (epilogue == kGemmEpiResAddF32 && (p_in.residual == nullptr || p_in.batch != 1)) return hipErrorInvalidValue;
+    if (epilogue == kGemmEpiRopeQkv && !gemm_f16_rope_supported(p_in)) return hipErrorInvalidValue;
     if (p_in.b2 != nullptr) {
         if (epilogue != kGemmEpiSiluGateF16 || !gemm_f16_dual_gate_supported(p_in)) return hipErrorInvalidValue;
         return launch_dma<kGemmEpiSiluGateF16, 4, 3, 64, 2, false, 2, true>(p_in, s); // 256 x 192 of both products, all of the LDS
@@ -778,6 +878,7 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         if (p.residual == nullptr || p.batch != 1) return hipErrorInvalidValue;
         return launch_dma_epi<kGemmEpiResAddF32>(p, tile, s);
     case kGemmEpiSiluGateF16: return launch_dma_epi<kGemmEpiSiluGateF16>(p, tile, s);
+    case kGemmEpiRopeQkv: return launch_dma_epi<kGemmEpiRopeQkv>(p, tile, s);
     default: return hipErrorInvalidValue;
     }
 }

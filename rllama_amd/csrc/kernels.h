@@ -99,12 +99,28 @@ hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s);
 size_t attn_decode_workspace_floats(int n_heads, int head_dim, int n_splits);
 constexpr int kAttnDecodeMaxSplits = 64;
 
+// What becomes of the wq|wk|wv product of a multi-token forward (prefill.hip; as an epilogue: gemm_dma.hip)
+struct PrefillRopeParams {
+    const void *qkv;        // [n x 3 dim] f16
+    const float2 *freqs;    // [max_seq_len x head_dim/2]
+    void *q_hi, *q_lo;      // [n_heads][n] rows of head_dim f16, q_stride halves apart
+    void *cache_k, *cache_v; // this layer: [n_heads][max_seq_len][head_dim]
+    int cache_f16;
+    void *v_t;              // [n_heads][head_dim][t_pad] f16
+    int n, dim, head_dim, max_seq_len, t_pad;
+    int q_stride;
+    int vt_swap;            // 1: positions within v_t rows have bits 2 and 3 swapped (the order attn_prefill_kernel reads)
+};
+
 // ---- prefill: C = A * B^T on the matrix cores (gemm.hip) ----
 enum GemmEpilogue {
     kGemmEpiF16 = 0,        // C f16 = round(acc)                      (projection outputs, tensor.rs:1623-1643)
     kGemmEpiF32 = 1,        // C f32 = acc, or += acc when accumulate  (attention scores / P.V partial products)
     kGemmEpiResAddF32 = 2,  // C f32 = residual + f16r(acc)            (wo and w2 followed by transformer.rs:442 / :445)
-    kGemmEpiSiluGateF16 = 3 // C f16 = round(silu(gate) * f16r(acc))   (w3 with w1's f16 output as the gate: transformer.rs:557-565)
+    kGemmEpiSiluGateF16 = 3, // C f16 = round(silu(gate) * f16r(acc))  (w3 with w1's f16 output as the gate: transformer.rs:557-565)
+    kGemmEpiRopeQkv = 4     // fast path only: the f16-rounded [m x 3 dim] product of wq|wk|wv is not stored; RoPE on its q and k
+                            // columns, q as hi + lo halves, k and v into the cache, v transposed (GemmParams::rope; what
+                            // rope_kv_prefill_tiled_kernel does with the stored product: transformer.rs:704-761)
 };
 
 struct GemmParams {
@@ -139,6 +155,7 @@ struct GemmParams {
     _Float16 *norm_out;     // [m x n], row stride n
     float norm_eps;
     int *norm_done;         // host flag
+    PrefillRopeParams rope; // kGemmEpiRopeQkv: the destinations (qkv unused; n = m, 3 dim = n, f16 cache, vt_swap as the reader expects)
 };
 
 hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s);
@@ -147,19 +164,10 @@ bool gemm_f16_dma_supported(const GemmParams &p);
 hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s);
 // whether the fast path runs w1 and w3 of a feed-forward block (b, b2: both [n x k]) as one pass over A for this shape
 bool gemm_f16_dual_gate_supported(const GemmParams &p);
+// whether the fast path applies RoPE and writes q / the cache / V^T straight from the wq|wk|wv product for this shape
+bool gemm_f16_rope_supported(const GemmParams &p);
 
 // ---- prefill: element-wise kernels around the GEMMs (prefill.hip) ----
-struct PrefillRopeParams {
-    const void *qkv;        // [n x 3 dim] f16
-    const float2 *freqs;    // [max_seq_len x head_dim/2]
-    void *q_hi, *q_lo;      // [n_heads][n] rows of head_dim f16, q_stride halves apart
-    void *cache_k, *cache_v; // this layer: [n_heads][max_seq_len][head_dim]
-    int cache_f16;
-    void *v_t;              // [n_heads][head_dim][t_pad] f16
-    int n, dim, head_dim, max_seq_len, t_pad;
-    int q_stride;
-    int vt_swap;            // 1: positions within v_t rows have bits 2 and 3 swapped (the order attn_prefill_kernel reads)
-};
 // fused causal attention of a multi-token forward (attn_prefill.hip); head_dim 64 or 128, f16 cache
 struct AttnPrefillParams {
     const void *q2;          // [n_heads][n] rows [q hi (head_dim) | q lo (head_dim)] f16, after RoPE

@@ -333,6 +333,35 @@ def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n):
     gm.free()
 
 
+@pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 384, 300), (128, 2, 256, 70), (64, 4, 128, 130), (192, 3, 256, 515), (512, 4, 640, 1024)])
+def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n):
+    """RoPE, the hi + lo halves of q, the cache rows and V^T written by the epilogue of the wq|wk|wv product (transformer.rs:
+    694-761 with seq_len > 1) against the same steps as a kernel of their own on the stored product: same values at the
+    same rounding points, so the same bits in the logits, in the token step that follows, and in every cache row.  Head
+    dimensions 128, 64 and 16 (the last takes the two-GEMM attention, which reads V^T in plain position order); ragged row
+    tiles; wavefront tiles that straddle the q | k and k | v column boundaries; and against the oracle."""
+    shape = Shape(dim=dim, n_layers=2, n_heads=heads, ffn_hidden=ffn, vocab_size=64, max_seq_len=n + 3)
+    W = synth_weights(shape, seed=71, std=0.05, norm_ones=False)
+    toks = np.random.default_rng(72).integers(0, shape.vocab_size, n + 1)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    got = {}
+    for mode in ("1", "0"):
+        os.environ["RLLAMA_HIP_GEMM_ROPE"] = mode
+        try:
+            gc = gm.make_caches()
+            a, b = gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc)
+            got[mode] = (a, b, [gc.read(l, h, w) for l in range(2) for h in range(heads) for w in (0, 1)])
+        finally:
+            del os.environ["RLLAMA_HIP_GEMM_ROPE"]
+    assert np.array_equal(got["1"][0], got["0"][0]) and np.array_equal(got["1"][1], got["0"][1])
+    for x, y in zip(got["1"][2], got["0"][2]):
+        assert np.array_equal(x, y)
+    oc = om.make_caches()
+    assert max_rel_err(got["1"][0], om.forward(toks[:n], 0, oc)) < TOL_F16
+    assert max_rel_err(got["1"][1], om.forward(toks[n:n + 1], n, oc)) < TOL_F16
+    gm.free()
+
+
 def test_prefill_long_prompt_causal_tiles(ctx):
     """A prompt long enough that the score matrix spans several GEMM tiles per head (tiles above the diagonal are
     skipped, the probability product stops at the diagonal) on the large-tile path; compared with the oracle."""
