@@ -785,25 +785,33 @@ static hipError_t launch_split_finish(const GemmParams &p, int splits, hipStream
     return hipGetLastError();
 }
 
-// Two products in one pass pay off where their workgroups (256 x 192 of both products each) fill the compute units about as
-// well as the best single-product tile does; shorter prompts keep the narrower tiles and split products of two launches.
-bool gemm_f16_dual_gate_supported(const GemmParams &p) {
-    const char *env = getenv("RLLAMA_HIP_GEMM_DUAL"); // 0: never, 1: wherever the kernel can run (tests), unset: by shape; read at every call
+// Two products in one pass pay off where their workgroups fill the compute units about as well as the best single-product
+// tile does.  Returns 0 (two launches), 1 (workgroups of 256 x 192 of both products, eight wavefronts, all of the LDS) or
+// 2 (128 x 192 of both, four wavefronts: prompts of about 300 to 512 rows, where the 128 x 128 tile of a single product needs two
+// rounds of workgroups and this form one).  The model is choose_tile's: rounds of workgroups x outputs per workgroup / relative
+// throughput of a busy compute unit, with 1.23 x 1.18 measured for the 256-row form (7B and 13B shapes, 256 to 2048 prompt
+// rows: faster from 768 rows on except where the last round is nearly empty) and 0.87 for the 128-row form (7B shape: 3 - 4 % of
+// the time to the first token at 384 and 512 rows, slower at 256 and 640).
+static int choose_dual(const GemmParams &p) {
+    const char *env = getenv("RLLAMA_HIP_GEMM_DUAL"); // 0: never, 1 / 2: that form wherever the kernel can run (tests), unset: by shape; read at every call
     const int mode = env != nullptr ? atoi(env) : -1;
-    if (mode == 0 || p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.k % 64 != 0) return false;
-    if ((p.ldc % 8) != 0 || (p.n % 8) != 0 || (reinterpret_cast<uintptr_t>(p.c) % 16) != 0) return false;
-    if (mode == 1) return true;
-    // the tile model of choose_tile: two launches of the best single tile against the rounds of 256 x 192 workgroups that do
-    // both products, whose busy compute unit measured 1.18 of the single 256 x 192 tile's throughput (7B and 13B shapes, 256 to
-    // 2048 prompt rows: faster from 768 rows on except where the last round is nearly empty, slower at 256)
+    if (mode == 0 || p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.k % 64 != 0) return 0;
+    if ((p.ldc % 8) != 0 || (p.n % 8) != 0 || (reinterpret_cast<uintptr_t>(p.c) % 16) != 0) return 0;
+    if (mode == 1 || mode == 2) return mode;
     double single = 0.0;
     const int tile = choose_tile(p, &single);
-    if (tile < 0 || tile > 3 || choose_split_k(p, tile) != 1) return false;
+    if (tile < 0 || tile > 3 || choose_split_k(p, tile) != 1) return 0;
     const int n_cu = device_compute_units();
-    const long blocks = (long)((p.n + 191) / 192) * ((p.m + 255) / 256);
-    const double dual = (double)((blocks + n_cu - 1) / n_cu) * 2.0 * 256 * 192 / (1.23 * 1.18);
-    return dual < 2.0 * single;
+    const long cols = (p.n + 191) / 192;
+    const long blocks256 = cols * ((p.m + 255) / 256), blocks128 = cols * ((p.m + 127) / 128);
+    const double dual256 = (double)((blocks256 + n_cu - 1) / n_cu) * 2.0 * 256 * 192 / (1.23 * 1.18);
+    const double dual128 = (double)((blocks128 + n_cu - 1) / n_cu) * 2.0 * 128 * 192 / 0.87;
+    const double best = dual256 <= dual128 ? dual256 : dual128;
+    if (best >= 2.0 * single) return 0;
+    return dual256 <= dual128 ? 1 : 2;
 }
+
+bool gemm_f16_dual_gate_supported(const GemmParams &p) { return choose_dual(p) != 0; }
 
 // The RoPE epilogue needs whole 16-byte pieces everywhere and an unsplit product (a product cut along K has its epilogue in
 // the kernel that adds the partial sums; the caller then stores the product and runs the separate kernel).
@@ -825,8 +833,10 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
     if (epilogue == kGemmEpiResAddF32 && (p_in.residual == nullptr || p_in.batch != 1)) return hipErrorInvalidValue;
     if (epilogue == kGemmEpiRopeQkv && !gemm_f16_rope_supported(p_in)) return hipErrorInvalidValue;
     if (p_in.b2 != nullptr) {
-        if (epilogue != kGemmEpiSiluGateF16 || !gemm_f16_dual_gate_supported(p_in)) return hipErrorInvalidValue;
-        return launch_dma<kGemmEpiSiluGateF16, 4, 3, 64, 2, false, 2, true>(p_in, s); // 256 x 192 of both products, all of the LDS
+        const int dual = epilogue == kGemmEpiSiluGateF16 ? choose_dual(p_in) : 0;
+        if (dual == 1) return launch_dma<kGemmEpiSiluGateF16, 4, 3, 64, 2, false, 2, true>(p_in, s); // 256 x 192 of both products, all of the LDS
+        if (dual == 2) return launch_dma<kGemmEpiSiluGateF16, 2, 3, 64, 2, false, 2, true>(p_in, s); // 128 x 192 of both, four wavefronts
+        return hipErrorInvalidValue;
     }
     if (epilogue == kGemmEpiSiluGateF16 && (p_in.gate == nullptr || p_in.batch != 1 || p_in.f32_operands)) return hipErrorInvalidValue;
     const int splits = choose_split_k(p_in, choose_tile(p_in));

@@ -191,13 +191,14 @@ def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
     want = (silu * u).astype(np.float16)
     X, W1, W3 = Tensor.from_numpy(ctx, x), Tensor.from_numpy(ctx, w1), Tensor.from_numpy(ctx, w3)
     got = {}
-    for mode in ("1", "0"):
+    for mode in ("1", "2", "0"):
         os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
         try:
             got[mode] = X.ffn_gate(W1, W3).to_numpy()
         finally:
             del os.environ["RLLAMA_HIP_GEMM_DUAL"]
     assert np.array_equal(got["1"].view(np.uint16), got["0"].view(np.uint16))
+    assert np.array_equal(got["2"].view(np.uint16), got["0"].view(np.uint16))
     one = got["1"]
     step = np.spacing(np.maximum(np.abs(want), np.abs(one))).astype(f32)
     assert np.mean(one != want) < 2e-2 and np.all(np.abs(one.astype(f32) - want.astype(f32)) <= 2 * step)

@@ -319,14 +319,15 @@ def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n):
     toks = np.random.default_rng(62).integers(0, shape.vocab_size, n + 1)
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
     got = {}
-    for mode in ("1", "0"):
+    for mode in ("1", "2", "0"):  # workgroups of 256 rows (eight wavefronts), of 128 rows (four), two launches
         os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
         try:
             gc = gm.make_caches()
             got[mode] = (gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc))
         finally:
             del os.environ["RLLAMA_HIP_GEMM_DUAL"]
-    assert np.array_equal(got["1"][0], got["0"][0]) and np.array_equal(got["1"][1], got["0"][1])
+    for mode in ("1", "2"):
+        assert np.array_equal(got[mode][0], got["0"][0]) and np.array_equal(got[mode][1], got["0"][1]), mode
     oc = om.make_caches()
     assert max_rel_err(got["1"][0], om.forward(toks[:n], 0, oc)) < TOL_F16
     assert max_rel_err(got["1"][1], om.forward(toks[n:n + 1], n, oc)) < TOL_F16
