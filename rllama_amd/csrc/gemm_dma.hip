@@ -877,6 +877,8 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         // weights; the pieces of a split product use it too
         if (p.m <= 128 && (p.batch == 1 || p.split_k > 1) && (long)((p.n + 127) / 128) * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = p.m <= 32 ? 6 : p.m <= 64 ? 7 : 5;
     }
+    // one 128 x 128 tile per workgroup it stays: the kernel whose wavefronts split the K-steps instead of the tile
+    if ((tile == 0 || tile == 4) && gemm_f16_kgroup_supported(p, epilogue)) return launch_gemm_f16_kgroup(p, epilogue, s);
     if (p.f32_operands) {
         if (epilogue != kGemmEpiF32 || ((p.k * 2) % 64) != 0 || (p.k_seg != 0 && ((p.k_seg * 2) % 64) != 0)) return hipErrorInvalidValue;
         return launch_dma_f32(p, tile, s);

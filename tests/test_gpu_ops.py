@@ -191,12 +191,14 @@ def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
     want = (silu * u).astype(np.float16)
     X, W1, W3 = Tensor.from_numpy(ctx, x), Tensor.from_numpy(ctx, w1), Tensor.from_numpy(ctx, w3)
     got = {}
+    os.environ["RLLAMA_HIP_GEMM_KGROUP"] = "0"  # the two-launch form on the kernel whose sum over k runs in the one-pass kernel's order
     for mode in ("1", "2", "0"):
         os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
         try:
             got[mode] = X.ffn_gate(W1, W3).to_numpy()
         finally:
             del os.environ["RLLAMA_HIP_GEMM_DUAL"]
+    del os.environ["RLLAMA_HIP_GEMM_KGROUP"]
     assert np.array_equal(got["1"].view(np.uint16), got["0"].view(np.uint16))
     assert np.array_equal(got["2"].view(np.uint16), got["0"].view(np.uint16))
     one = got["1"]

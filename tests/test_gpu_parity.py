@@ -309,7 +309,7 @@ def test_prefill_wide_ffn_largest_tile(ctx):
 
 
 @pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 1000, 300), (128, 2, 192, 256), (192, 3, 1544, 515)])
-def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n):
+def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n, monkeypatch):
     """w1 and w3 as one pass over the normalised rows (two accumulator sets per wavefront, SiLU(w1 x) * (w3 x) straight from
     them: transformer.rs:551-565), forced onto shapes the oracle handles quickly: ragged last row and column tiles (300 and
     515 rows on 256-row tiles, 1000 = 5 x 192 + 40 and 1544 = 8 x 192 + 8 columns), exactly one tile, three K-tiles.  Same
@@ -319,6 +319,8 @@ def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n):
     toks = np.random.default_rng(62).integers(0, shape.vocab_size, n + 1)
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
     got = {}
+    # (the two-launch form on the tile-splitting kernel, whose sum over k runs in the same order as the one-pass kernel's)
+    monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", "0")
     for mode in ("1", "2", "0"):  # workgroups of 256 rows (eight wavefronts), of 128 rows (four), two launches
         os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
         try:
@@ -335,7 +337,7 @@ def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n):
 
 
 @pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 384, 300), (128, 2, 256, 70), (64, 4, 128, 130), (192, 3, 256, 515), (512, 4, 640, 1024)])
-def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n):
+def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n, monkeypatch):
     """RoPE, the hi + lo halves of q, the cache rows and V^T written by the epilogue of the wq|wk|wv product (transformer.rs:
     694-761 with seq_len > 1) against the same steps as a kernel of their own on the stored product: same values at the
     same rounding points, so the same bits in the logits, in the token step that follows, and in every cache row.  Head
@@ -346,6 +348,8 @@ def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n)
     toks = np.random.default_rng(72).integers(0, shape.vocab_size, n + 1)
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
     got = {}
+    # (the stored product on the tile-splitting kernel, whose sum over k runs in the same order as the kernel with the epilogue)
+    monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", "0")
     for mode in ("1", "0"):
         os.environ["RLLAMA_HIP_GEMM_ROPE"] = mode
         try:
@@ -360,6 +364,28 @@ def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n)
     oc = om.make_caches()
     assert max_rel_err(got["1"][0], om.forward(toks[:n], 0, oc)) < TOL_F16
     assert max_rel_err(got["1"][1], om.forward(toks[n:n + 1], n, oc)) < TOL_F16
+    gm.free()
+
+
+@pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 704, 300), (512, 4, 1408, 520), (128, 2, 192, 130)])
+def test_prefill_k_steps_split_among_wavefronts(ctx, dim, heads, ffn, n, monkeypatch):
+    """wo and w2 (and the other projections at these sizes) on the kernel whose wavefronts split the K-steps of a 128 x 128 tile
+    and add their four partial sums through LDS: against the oracle, and close to the tile-splitting kernel (the order of the
+    fp32 additions differs, so single f16 rounding decisions may)."""
+    shape = Shape(dim=dim, n_layers=2, n_heads=heads, ffn_hidden=ffn, vocab_size=64, max_seq_len=n + 2)
+    W = synth_weights(shape, seed=81, std=0.05, norm_ones=False)
+    toks = np.random.default_rng(82).integers(0, shape.vocab_size, n + 1)
+    om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
+    got = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", mode)
+        gc = gm.make_caches()
+        got[mode] = (gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc))
+    oc = om.make_caches()
+    want = (om.forward(toks[:n], 0, oc), om.forward(toks[n:n + 1], n, oc))
+    for i in (0, 1):
+        assert max_rel_err(got["1"][i], want[i]) < TOL_F16
+        assert max_rel_err(got["1"][i], got["0"][i]) < 2e-3
     gm.free()
 
 
@@ -739,9 +765,13 @@ def test_layer_span_on_a_whole_model_equals_its_forward(ctx):
 # the last four are sized so that the tile choice lands on the 256 x 192, 256 x 256 and 256 x 128 tiles (with ragged edges)
 @pytest.mark.parametrize("n,m_rows,k", [(2, 3, 8), (33, 65, 72), (128, 128, 64), (130, 200, 192), (16, 2816, 1024), (257, 384, 4096), (1024, 256, 11008),
                                         (1024, 12288, 64), (1000, 12290, 160), (1024, 16384, 96), (512, 16384, 96)])
-def test_mfma_gemm_f16(ctx, n, m_rows, k):
+@pytest.mark.parametrize("kgroup", ["1", "0"], ids=["k-steps-split", "tile-split"])
+def test_mfma_gemm_f16(ctx, n, m_rows, k, kgroup, monkeypatch):
     """src [n x k] . other[m x k]^T with n > 1 runs on the matrix cores; every element against the oracle's
-    f16-rounded dot8 (tensor.rs:1476-1666), including tiles that straddle the matrix edges."""
+    f16-rounded dot8 (tensor.rs:1476-1666), including tiles that straddle the matrix edges.  Products that take 128 x 128
+    tiles with k a multiple of 64 run on the kernel whose wavefronts split the K-steps of a tile (four partial sums per
+    element, added in a fixed order) unless that is switched off; both forms are checked."""
+    monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", kgroup)
     rng = np.random.default_rng(n * 7 + m_rows * 3 + k)
     a = oracle.f32_to_f16_bits(rng.uniform(-1, 1, (n, k)).astype(f32))
     b = oracle.f32_to_f16_bits((rng.standard_normal((m_rows, k)) * 0.05).astype(f32))
