@@ -17,6 +17,7 @@
 // on K ranges whose partial sums gemm_split_finish_kernel adds up (both further down).
 #include "kernels.h"
 #include "device_utils.h"
+#include "gemm_epilogue.h"
 
 #include <cstdlib>
 
@@ -390,7 +391,6 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
         constexpr int kPad = (kWaves * kWR * (kTW + 8) * 2 <= kStages * kStageBytes) ? 8 : 0;
         constexpr int kTS = kTW + kPad;
         static_assert(kWaves * kWR * kTS * 2 <= kStages * kStageBytes, "the output tiles reuse the stages");
-        constexpr int kChunks = kTW / 8;
         __syncthreads(); // every wavefront has read its last fragments
         half_t *tile = reinterpret_cast<half_t *>(lds_raw) + wave * (kWR * kTS);
 #pragma unroll
@@ -399,67 +399,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
             for (int j = 0; j < kNT; j++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) tile[(i * 32 + (v >> 2) * 8 + row_in + (v & 3)) * kTS + j * 32 + col_in] = (half_t)acc[i][j][v];
-        const int d = R.dim, hd = R.head_dim, half_hd = hd / 2;
-        half_t *qhi = reinterpret_cast<half_t *>(R.q_hi), *qlo = reinterpret_cast<half_t *>(R.q_lo);
-        half_t *ck = reinterpret_cast<half_t *>(R.cache_k), *cv = reinterpret_cast<half_t *>(R.cache_v);
-        const int wr0 = bm0 + wm * kWR, wc0 = bn0 + wn * kTW; // first row (position) and column of this wavefront's tile
-#pragma unroll
-        for (int it = 0; it < kChunks * kWR / 64; it++) {
-            const int idx = it * 64 + lane;
-            const int rr = idx / kChunks, ch = idx - rr * kChunks;
-            const int r = wr0 + rr, c = wc0 + ch * 8;
-            if (r < M && c < N) {
-                const half8_t o = *reinterpret_cast<const half8_t *>(tile + rr * kTS + ch * 8);
-                const int part = c / d, cin = c - part * d; // 0 q, 1 k, 2 v
-                const int head = cin / hd, d0 = cin - head * hd;
-                const size_t co = ((size_t)head * R.max_seq_len + r) * hd + d0;
-                if (part == 2) {
-                    *reinterpret_cast<half8_t *>(cv + co) = o;
-                } else {
-                    const float2 *fr = R.freqs + (size_t)r * half_hd + d0 / 2;
-                    half8_t hi, lo;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        float a, b;
-                        rope_pair((float)o[2 * e], (float)o[2 * e + 1], fr[e], a, b);
-                        hi[2 * e] = (half_t)a;
-                        hi[2 * e + 1] = (half_t)b;
-                        lo[2 * e] = (half_t)(a - (float)hi[2 * e]);
-                        lo[2 * e + 1] = (half_t)(b - (float)hi[2 * e + 1]);
-                    }
-                    if (part == 0) {
-                        const size_t qo = ((size_t)head * M + r) * R.q_stride + d0;
-                        *reinterpret_cast<half8_t *>(qhi + qo) = hi;
-                        *reinterpret_cast<half8_t *>(qlo + qo) = lo;
-                    } else {
-                        *reinterpret_cast<half8_t *>(ck + co) = hi; // the rotated k rounded to f16
-                    }
-                }
-            }
-        }
-        // V^T [dim][t_pad]: 8 consecutive (stored) positions of one column per piece; eight lanes cover the 64 positions of a
-        // column, i.e. 128 contiguous bytes.  Rows past m hold copies of the last row (finite), which is what the padding of
-        // V^T needs.  With vt_swap the stored order within every 16 positions has bits 2 and 3 of the position exchanged.
-        if (wc0 + kTW > 2 * d) {
-            half_t *vt = reinterpret_cast<half_t *>(R.v_t);
-            constexpr int kPieces = kWR / 8;
-#pragma unroll
-            for (int it = 0; it < kTW * kPieces / 64; it++) {
-                const int idx = it * 64 + lane;
-                const int cc = idx / kPieces, j = idx - cc * kPieces;
-                const int c = wc0 + cc, pos0 = wr0 + j * 8;
-                if (c >= 2 * d && c < N && pos0 < R.t_pad) {
-                    half8_t o;
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const int rs = j * 8 + e;
-                        const int src = R.vt_swap ? (rs & ~12) | ((rs & 4) << 1) | ((rs & 8) >> 1) : rs;
-                        o[e] = tile[src * kTS + cc];
-                    }
-                    *reinterpret_cast<half8_t *>(vt + (size_t)(c - 2 * d) * R.t_pad + pos0) = o;
-                }
-            }
-        }
+        rope_qkv_from_tile<kWR, kTW, kTS>(tile, lane, bm0 + wm * kWR, bn0 + wn * kTW, M, N, R);
         return;
     }
     if constexpr (kEpi == kGemmEpiF16 || kEpi == kGemmEpiSiluGateF16) {
@@ -642,7 +582,11 @@ static int choose_tile(const GemmParams &p, double *model_time = nullptr) {
     if (forced == 0 && k_halves % 64 == 0) return 0;
     const int n_cu = device_compute_units();
     const int bms[4] = {128, 256, 256, 256}, bns[4] = {128, 128, 192, 256};
-    const double eff[4] = {1.0, 1.05, 1.23, 1.15}; // relative throughput of a busy compute unit, measured on 7B shapes
+    // relative throughput of a busy compute unit, measured on 7B shapes.  (The 128 x 128 tile of the kernel whose wavefronts
+    // split the K-steps, gemm_kgroup.hip, is 1.15 in one round of workgroups, but rating it so here sends products to it in
+    // two and three rounds, where it loses: 7B shape 1536 / 2048 rows 26.1 / 30.0 ms to the first token against 24.7 / 28.9,
+    // 13B shape 1024 rows 35.6 against 31.2.  It takes over only where this model picks the 128 x 128 tile anyway.)
+    const double eff[4] = {1.0, 1.05, 1.23, 1.15};
     int best = -1;
     double best_t = 0.0;
     for (int t = 0; t < 4; t++) {
@@ -877,8 +821,8 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         // weights; the pieces of a split product use it too
         if (p.m <= 128 && (p.batch == 1 || p.split_k > 1) && (long)((p.n + 127) / 128) * 2 <= device_compute_units() && p.k_seg == 0 && p.causal == 0) tile = p.m <= 32 ? 6 : p.m <= 64 ? 7 : 5;
     }
-    // one 128 x 128 tile per workgroup it stays: the kernel whose wavefronts split the K-steps instead of the tile
-    if ((tile == 0 || tile == 4) && gemm_f16_kgroup_supported(p, epilogue)) return launch_gemm_f16_kgroup(p, epilogue, s);
+    // 128 x 128 or 256 x 192 per workgroup it stays: the kernel whose wavefronts split the K-steps instead of the tile
+    if (gemm_f16_kgroup_supported(p, epilogue, tile)) return launch_gemm_f16_kgroup(p, epilogue, tile, s);
     if (p.f32_operands) {
         if (epilogue != kGemmEpiF32 || ((p.k * 2) % 64) != 0 || (p.k_seg != 0 && ((p.k_seg * 2) % 64) != 0)) return hipErrorInvalidValue;
         return launch_dma_f32(p, tile, s);

@@ -166,8 +166,8 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p, int epilogue, hipStream_t s)
 bool gemm_f16_dual_gate_supported(const GemmParams &p);
 // small output tiles per compute unit (gemm_kgroup.hip): wavefronts split the K-steps instead of the tile; launch_gemm_f16_dma
 // hands such products over
-bool gemm_f16_kgroup_supported(const GemmParams &p, int epilogue);
-hipError_t launch_gemm_f16_kgroup(const GemmParams &p, int epilogue, hipStream_t s);
+bool gemm_f16_kgroup_supported(const GemmParams &p, int epilogue, int tile);
+hipError_t launch_gemm_f16_kgroup(const GemmParams &p, int epilogue, int tile, hipStream_t s);
 // whether the fast path applies RoPE and writes q / the cache / V^T straight from the wq|wk|wv product for this shape
 bool gemm_f16_rope_supported(const GemmParams &p);
 
