@@ -35,9 +35,7 @@ constexpr int kgroup_round_tiles(int n_waves, int kg, int nt, int lds_bytes) {
 }
 
 // kWM x kWN wavefront tiles of (32 kIT) x (32 kNT) per K-group, kKG K-groups: kWM kWN kKG wavefronts.
-// kLean: the A fragments are single-buffered (the MFMAs of a K-step run row slab by row slab, and a slab's fragment is
-// replaced by the next K-step's as soon as its MFMAs are issued), for tiles whose accumulators leave no room for two sets.
-template <int kEpi, int kWM, int kWN, int kKG, int kIT, int kNT, int kStages, bool kLean = false>
+template <int kEpi, int kWM, int kWN, int kKG, int kIT, int kNT, int kStages>
 __global__ __launch_bounds__(64 * kWM * kWN * kKG) void gemm_f16_kgroup_kernel(GemmParams p) {
     constexpr int kBK = 64, kKS = kBK / 16, kMy = kKS / kKG;
     static_assert(kKS % kKG == 0 && kIT % kKG == 0, "K-steps and row slabs divide among the K-groups");
@@ -130,20 +128,14 @@ __global__ __launch_bounds__(64 * kWM * kWN * kKG) void gemm_f16_kgroup_kernel(G
     int coff[kMy]; // byte offset of this wavefront's s-th K-step within a row
 #pragma unroll
     for (int s = 0; s < kMy; s++) coff[s] = (((s * kKG + g) * 2 + fch) ^ sw) << 4;
-    half8_t fa[kLean ? 1 : 2][kIT], fb[2][kNT];
-    auto read_a = [&](int set, int i, const unsigned char *stage, int s) {
-        fa[kLean ? 0 : set][i] = *reinterpret_cast<const half8_t *>(stage + xa + i * (32 * kRowBytes) + coff[s]);
-    };
-    auto read_b = [&](int set, const unsigned char *stage, int s) {
+    half8_t fa[2][kIT], fb[2][kNT];
+    auto read_frags = [&](int set, const unsigned char *stage, int s) {
+#pragma unroll
+        for (int i = 0; i < kIT; i++) fa[set][i] = *reinterpret_cast<const half8_t *>(stage + xa + i * (32 * kRowBytes) + coff[s]);
 #pragma unroll
         for (int j = 0; j < kNT; j++) fb[set][j] = *reinterpret_cast<const half8_t *>(stage + xb + j * (32 * kRowBytes) + coff[s]);
     };
-    auto read_frags = [&](int set, const unsigned char *stage, int s) {
-#pragma unroll
-        for (int i = 0; i < kIT; i++) read_a(set, i, stage, s);
-        read_b(set, stage, s);
-    };
-    auto mma = [&](int set, int i, int j) { acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kLean ? 0 : set][i], fb[set][j], acc[i][j], 0, 0, 0); };
+    auto mma = [&](int set, int i, int j) { acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0); };
 
     // Software pipeline as in gemm_dma.hip: all stages in flight at the start; the fragments of a wavefront's next K-step are
     // read while the MFMAs of the current one run; the K-tile change (wait, barrier, refill, first fragments of the next tile)
@@ -159,37 +151,7 @@ __global__ __launch_bounds__(64 * kWM * kWN * kKG) void gemm_f16_kgroup_kernel(G
 #pragma unroll
         for (int s = 0; s < kMy; s++) {
             const int cur = (decltype(parity)::value * kMy + s) & 1, nxt = cur ^ 1;
-            if constexpr (kLean) {
-                if (s + 1 < kMy) {
-                    read_b(nxt, stage, s + 1);
-#pragma unroll
-                    for (int i = 0; i < kIT; i++) {
-#pragma unroll
-                        for (int j = 0; j < kNT; j++) mma(cur, i, j);
-                        read_a(nxt, i, stage, s + 1);
-                    }
-                } else {
-                    const unsigned char *next = lds_raw + ((kt + 1) % kStages) * kStageBytes;
-#pragma unroll
-                    for (int i = 0; i < kIT / 2; i++)
-#pragma unroll
-                        for (int j = 0; j < kNT; j++) mma(cur, i, j);
-                    __builtin_amdgcn_sched_barrier(0);
-                    wait_vmcnt<(kStages - 2) * kLoads>();
-                    __syncthreads(); // K-tile kt + 1 is in LDS for everybody, and nobody reads K-tile kt any more
-                    issue(kt + kStages);
-                    read_b(nxt, next, 0);
-#pragma unroll
-                    for (int i = 0; i < kIT / 2; i++) read_a(nxt, i, next, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int i = kIT / 2; i < kIT; i++) {
-#pragma unroll
-                        for (int j = 0; j < kNT; j++) mma(cur, i, j);
-                        read_a(nxt, i, next, 0);
-                    }
-                }
-            } else if (s + 1 < kMy) {
+            if (s + 1 < kMy) {
                 read_frags(nxt, stage, s + 1);
 #pragma unroll
                 for (int j = 0; j < kNT; j++)
@@ -335,7 +297,7 @@ bool gemm_f16_kgroup_supported(const GemmParams &p, int epilogue, int tile) {
     const char *env = getenv("RLLAMA_HIP_GEMM_KGROUP"); // 0: never; read at every call
     if (env != nullptr && atoi(env) == 0) return false;
     // tile: the choice of gemm_dma.hip's model -- 0 / 4: 128 x 128.  (256 x 192 tiles with wavefronts of 128 x 96 on every other
-    // K-step -- kLean, 192 accumulator registers -- measured 98.8 against 102.2 us on the plain wq|wk|wv product of the 7B shape
+    // K-step -- 192 accumulator registers, A fragments single-buffered -- measured 98.8 against 102.2 us on the plain wq|wk|wv product of the 7B shape
     // and 112.4 against 111 us with RoPE and the cache write in the epilogue: the cycles fall as the LDS bytes do, the clock
     // falls with them (power), and the exchange of the partial sums is added.  Not wired in.)
     if (tile != 0 && tile != 4) return false;
@@ -346,16 +308,16 @@ bool gemm_f16_kgroup_supported(const GemmParams &p, int epilogue, int tile) {
     return true;
 }
 
-template <int kEpi, int kWM, int kWN, int kKG, int kIT, int kNT, int kStages, bool kLean>
+template <int kEpi, int kWM, int kWN, int kKG, int kIT, int kNT, int kStages>
 static hipError_t launch_kgroup(const GemmParams &p, hipStream_t s) {
     constexpr int bm = 32 * kIT * kWM, bn = 32 * kNT * kWN;
     constexpr size_t lds = (size_t)kStages * (bm + bn) * 64 * 2;
     static_assert(lds <= 160 * 1024, "LDS of one compute unit");
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_kgroup_kernel<kEpi, kWM, kWN, kKG, kIT, kNT, kStages, kLean>),
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_kgroup_kernel<kEpi, kWM, kWN, kKG, kIT, kNT, kStages>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) return attr;
     const dim3 grid((p.n + bn - 1) / bn, (p.m + bm - 1) / bm, 1);
-    hipLaunchKernelGGL((gemm_f16_kgroup_kernel<kEpi, kWM, kWN, kKG, kIT, kNT, kStages, kLean>), grid, dim3(64 * kWM * kWN * kKG), lds, s, p);
+    hipLaunchKernelGGL((gemm_f16_kgroup_kernel<kEpi, kWM, kWN, kKG, kIT, kNT, kStages>), grid, dim3(64 * kWM * kWN * kKG), lds, s, p);
     return hipGetLastError();
 }
 
@@ -364,8 +326,8 @@ hipError_t launch_gemm_f16_kgroup(const GemmParams &p, int epilogue, int tile, h
     // 128 x 128 per workgroup: eight wavefronts = two column halves x four K-groups, each wavefront on 128 x 64 for one K-step in
     // four (the whole tile per wavefront -- 256 accumulator registers -- does not survive hipcc's register allocation); four
     // stages of 32 KB
-    if (epilogue == kGemmEpiF16) return launch_kgroup<kGemmEpiF16, 1, 2, 4, 4, 2, 4, false>(p, s);
-    return launch_kgroup<kGemmEpiResAddF32, 1, 2, 4, 4, 2, 4, false>(p, s);
+    if (epilogue == kGemmEpiF16) return launch_kgroup<kGemmEpiF16, 1, 2, 4, 4, 2, 4>(p, s);
+    return launch_kgroup<kGemmEpiResAddF32, 1, 2, 4, 4, 2, 4>(p, s);
 }
 
 } // namespace rlh
