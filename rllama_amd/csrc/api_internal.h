@@ -32,7 +32,9 @@ struct OpScratch {
     size_t attn_ws_floats = 0;
     unsigned *tickets = nullptr;   // [kOpMaxHeads]
     int32_t *token = nullptr;      // one id
+    void *gemm_ws = nullptr;       // partial sums of products cut along K (kOpGemmWsBytes), as the forward's prompt path has
 };
+constexpr size_t kOpGemmWsBytes = (size_t)64 << 20;
 constexpr int kOpMaxHeads = 1024;
 
 struct rlh_ctx {

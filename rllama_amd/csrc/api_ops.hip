@@ -199,6 +199,9 @@ extern "C" int rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tens
         g.ldc = mrows;
         g.batch = 1;
         g.f32_operands = f16 ? 0 : 1;
+        if (!dst->ctx->ops.gemm_ws) HIP_TRY(hipMalloc(&dst->ctx->ops.gemm_ws, kOpGemmWsBytes));
+        g.workspace = dst->ctx->ops.gemm_ws;
+        g.workspace_bytes = kOpGemmWsBytes;
         HIP_TRY(launch_gemm_f16(g, f16 ? kGemmEpiF16 : kGemmEpiF32, st));
         return RLH_OK;
     }
@@ -296,6 +299,9 @@ extern "C" int rlh_ffn_gate(rlh_tensor *dst, const rlh_tensor *x, const rlh_tens
     g.lda = g.ldb = x->cols;
     g.ldc = w1->rows;
     g.batch = 1;
+    if (!dst->ctx->ops.gemm_ws) HIP_TRY(hipMalloc(&dst->ctx->ops.gemm_ws, kOpGemmWsBytes));
+    g.workspace = dst->ctx->ops.gemm_ws;
+    g.workspace_bytes = kOpGemmWsBytes;
     GemmParams both = g;
     both.b2 = (const _Float16 *)w3->p;
     if (gemm_f16_dual_gate_supported(both)) { // both products in one pass over x
@@ -394,7 +400,7 @@ static int ensure_op_scratch(rlh_ctx *ctx, size_t attn_ws_floats) {
 namespace rlh {
 void ops_release(rlh_ctx *ctx) {
     OpScratch &o = ctx->ops;
-    void *all[] = {o.state, o.attn_ws, o.tickets, o.token};
+    void *all[] = {o.state, o.attn_ws, o.tickets, o.token, o.gemm_ws};
     for (void *b : all)
         if (b) (void)hipFree(b);
     o = OpScratch();

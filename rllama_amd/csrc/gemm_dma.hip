@@ -614,13 +614,13 @@ static int choose_tile(const GemmParams &p, double *model_time = nullptr) {
 // Second step of a split-K product: C = epilogue(sum over the split_k partial sums, in the order of the splits).
 template <int kEpi>
 __global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int splits) {
-    const size_t per = (size_t)p.m * p.ldc;
-    const int n4 = p.n / 4; // n is a multiple of 4 here
+    const size_t per = (size_t)p.m * p.n; // the partial sums are [splits][m][n], n a multiple of 4 here
+    const int n4 = p.n / 4;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (size_t)p.m * n4; i += (size_t)gridDim.x * blockDim.x) {
         const int r = (int)(i / n4), c = (int)(i % n4) * 4;
-        const size_t off = (size_t)r * p.ldc + c;
-        float4_t acc = *reinterpret_cast<const float4_t *>(partial + off);
-        for (int z = 1; z < splits; z++) acc += *reinterpret_cast<const float4_t *>(partial + z * per + off);
+        const size_t off = (size_t)r * p.ldc + c, woff = i * 4;
+        float4_t acc = *reinterpret_cast<const float4_t *>(partial + woff);
+        for (int z = 1; z < splits; z++) acc += *reinterpret_cast<const float4_t *>(partial + z * per + woff);
         if constexpr (kEpi == kGemmEpiF16) {
             typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
             half4_t o;
@@ -656,9 +656,9 @@ __global__ void gemm_split_finish_kernel(GemmParams p, const float *partial, int
 constexpr int kFinishNormVecs = 8; // rows of up to 256 x 4 x 8 floats
 __global__ __launch_bounds__(256) void gemm_split_finish_norm_kernel(GemmParams p, const float *partial, int splits) {
     __shared__ float red[16];
-    const size_t per = (size_t)p.m * p.ldc;
+    const size_t per = (size_t)p.m * p.n;
     const int r = blockIdx.x, tid = threadIdx.x, n4 = p.n / 4;
-    const size_t row = (size_t)r * p.ldc;
+    const size_t row = (size_t)r * p.ldc, wrow = (size_t)r * p.n;
     const float4_t *w4 = reinterpret_cast<const float4_t *>(p.norm_w);
     float4_t xv[kFinishNormVecs];
     float ss = 0.0f;
@@ -667,9 +667,9 @@ __global__ __launch_bounds__(256) void gemm_split_finish_norm_kernel(GemmParams 
         const int i = tid + j * 256;
         xv[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
         if (i < n4) {
-            const size_t off = row + (size_t)i * 4;
-            float4_t acc = *reinterpret_cast<const float4_t *>(partial + off);
-            for (int z = 1; z < splits; z++) acc += *reinterpret_cast<const float4_t *>(partial + z * per + off);
+            const size_t off = row + (size_t)i * 4, woff = wrow + (size_t)i * 4;
+            float4_t acc = *reinterpret_cast<const float4_t *>(partial + woff);
+            for (int z = 1; z < splits; z++) acc += *reinterpret_cast<const float4_t *>(partial + z * per + woff);
             const float4_t res = *reinterpret_cast<const float4_t *>(p.residual + off);
 #pragma unroll
             for (int e = 0; e < 4; e++) xv[j][e] = res[e] + f16r(acc[e]);
@@ -716,7 +716,7 @@ static int choose_split_k(const GemmParams &p, int tile) {
     const long tiles = p.m <= 128 ? (long)((p.n + 63) / 64) : blocks;
     long s = forced > 1 ? forced : (n_cu + tiles - 1) / tiles;
     if (s > k_tiles / 4) s = k_tiles / 4;                  // at least 4 K-tiles per piece
-    const size_t per = (size_t)p.m * p.ldc * sizeof(float);
+    const size_t per = (size_t)p.m * p.n * sizeof(float);
     if (per > 0 && (size_t)s * per > p.workspace_bytes) s = (long)(p.workspace_bytes / per);
     return s < 2 ? 1 : (int)s;
 }
@@ -792,7 +792,8 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         q.split_k = splits;
         q.batch = splits;
         q.stride_a = q.stride_b = 0;
-        q.stride_c = (size_t)p_in.m * p_in.ldc;
+        q.ldc = p_in.n;
+        q.stride_c = (size_t)p_in.m * p_in.n;
         q.workspace = nullptr;
         hipError_t e = launch_gemm_f16_dma(q, kGemmEpiF32, s);
         if (e != hipSuccess) return e;

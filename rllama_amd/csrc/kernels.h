@@ -143,7 +143,7 @@ struct GemmParams {
                             // 2: of every segment only k < (last row of the C tile) + 1, rounded up to the K-tile, is used
                             //    (A holds zeros beyond the diagonal: causal probabilities times V)
     int split_k;            // set by the launcher only: grid.z = K ranges of one product (see gemm_dma.hip)
-    void *workspace;        // optional, for split-K partial sums: fp32 [pieces][m][ldc]; without it products run unsplit
+    void *workspace;        // optional, for split-K partial sums: fp32 [pieces][m][n rounded up to 4]; without it products run unsplit
     size_t workspace_bytes;
     int f32_operands;       // 1: a and b point to fp32 data (f32 mode); m, n, k, lda, ldb, strides and k_seg count elements
                             //    all the same.  Needs k % 32 == 0 and the kGemmEpiF32 epilogue.
