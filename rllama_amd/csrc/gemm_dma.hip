@@ -662,21 +662,45 @@ __global__ __launch_bounds__(256) void gemm_split_finish_norm_kernel(GemmParams 
     const float4_t *w4 = reinterpret_cast<const float4_t *>(p.norm_w);
     float4_t xv[kFinishNormVecs];
     float ss = 0.0f;
+    // the pieces outermost, so that a thread's loads of one piece are all in flight together (per element the partial sums are
+    // still added in the order of the pieces)
 #pragma unroll
     for (int j = 0; j < kFinishNormVecs; j++) {
         const int i = tid + j * 256;
-        xv[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        if (i < n4) {
-            const size_t off = row + (size_t)i * 4, woff = wrow + (size_t)i * 4;
-            float4_t acc = *reinterpret_cast<const float4_t *>(partial + woff);
-            for (int z = 1; z < splits; z++) acc += *reinterpret_cast<const float4_t *>(partial + z * per + woff);
-            const float4_t res = *reinterpret_cast<const float4_t *>(p.residual + off);
+        xv[j] = i < n4 ? *reinterpret_cast<const float4_t *>(partial + wrow + (size_t)i * 4) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    float4_t res[kFinishNormVecs];
 #pragma unroll
-            for (int e = 0; e < 4; e++) xv[j][e] = res[e] + f16r(acc[e]);
-            *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.c) + off) = xv[j];
+    for (int j = 0; j < kFinishNormVecs; j++) {
+        const int i = tid + j * 256;
+        res[j] = i < n4 ? *reinterpret_cast<const float4_t *>(p.residual + row + (size_t)i * 4) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    for (int z = 1; z < splits; z++) {
+        float4_t part[kFinishNormVecs];
+#pragma unroll
+        for (int j = 0; j < kFinishNormVecs; j++) {
+            const int i = tid + j * 256;
+            part[j] = i < n4 ? *reinterpret_cast<const float4_t *>(partial + z * per + wrow + (size_t)i * 4) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+#pragma unroll
+        for (int j = 0; j < kFinishNormVecs; j++) xv[j] += part[j];
+    }
+#pragma unroll
+    for (int j = 0; j < kFinishNormVecs; j++) {
+        const int i = tid + j * 256;
+        if (i < n4) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) xv[j][e] = res[j][e] + f16r(xv[j][e]);
+            *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.c) + row + (size_t)i * 4) = xv[j];
         }
 #pragma unroll
         for (int e = 0; e < 4; e++) ss = fmaf(xv[j][e], xv[j][e], ss);
+    }
+    float4_t wn[kFinishNormVecs]; // requested before the row sum, not after it
+#pragma unroll
+    for (int j = 0; j < kFinishNormVecs; j++) {
+        const int i = tid + j * 256;
+        wn[j] = i < n4 ? w4[i] : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
     ss = block_sum(ss, red);
     const float rs = 1.0f / sqrtf(ss / (float)p.n + p.norm_eps);
@@ -685,7 +709,7 @@ __global__ __launch_bounds__(256) void gemm_split_finish_norm_kernel(GemmParams 
     for (int j = 0; j < kFinishNormVecs; j++) {
         const int i = tid + j * 256;
         if (i < n4) {
-            const float4_t wv = w4[i];
+            const float4_t wv = wn[j];
             typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
             half4_t o;
 #pragma unroll

@@ -47,13 +47,19 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_f16_kernel(half_t *y, const 
 #pragma unroll
             for (int e = 0; e < 4; e++) ss = fmaf(xv[j][e], xv[j][e], ss);
         }
+        float4_t wn[kNormVecs]; // requested before the row sum, not after it
+#pragma unroll
+        for (int j = 0; j < kNormVecs; j++) {
+            const int i = tid + j * 256;
+            wn[j] = i < n4 ? w4[i] : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
         ss = block_sum(ss, red);
         const float rs = 1.0f / sqrtf(ss / (float)d + eps);
 #pragma unroll
         for (int j = 0; j < kNormVecs; j++) {
             const int i = tid + j * 256;
             if (i < n4) {
-                const float4_t wv = w4[i];
+                const float4_t wv = wn[j];
                 typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
                 half4_t o;
 #pragma unroll
