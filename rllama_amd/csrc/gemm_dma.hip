@@ -290,7 +290,7 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
                 }
-                __builtin_amdgcn_sched_group_barrier(0x008, kIT * kNT - kNT, 0);
+                if constexpr (kIT * kNT - kNT > 0) __builtin_amdgcn_sched_group_barrier(0x008, kIT * kNT - kNT, 0);
                 if (ks + 1 < kKS) {
                     read_a(nxt, stage, ks + 1);
                     read_b(b0, stage, ks + 1, 0);
@@ -298,12 +298,14 @@ __global__ __launch_bounds__(128 * kWavesM) void gemm_f16_dma_kernel(GemmParams 
                     for (int j = 0; j < kNT; j++)
 #pragma unroll
                         for (int i = 0; i < kIT; i++) mma(af[cur][i], b1[j], acc[i][kNT + j]);
+                    constexpr int kMmas2 = kIT * kNT, kReads2 = kIT + kNT, kPairs2 = kMmas2 < kReads2 ? kMmas2 : kReads2;
 #pragma unroll
-                    for (int r = 0; r < kIT + kNT; r++) {
+                    for (int r = 0; r < kPairs2; r++) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                     }
-                    __builtin_amdgcn_sched_group_barrier(0x008, kIT * kNT - (kIT + kNT), 0);
+                    if constexpr (kMmas2 > kPairs2) __builtin_amdgcn_sched_group_barrier(0x008, kMmas2 - kPairs2, 0);
+                    if constexpr (kReads2 > kPairs2) __builtin_amdgcn_sched_group_barrier(0x100, kReads2 - kPairs2, 0);
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
                     wait_vmcnt<(kStages - 2) * kLoads>();
@@ -754,18 +756,27 @@ static hipError_t launch_split_finish(const GemmParams &p, int splits, hipStream
 }
 
 // Two products in one pass pay off where their workgroups fill the compute units about as well as the best single-product
-// tile does.  Returns 0 (two launches), 1 (workgroups of 256 x 192 of both products, eight wavefronts, all of the LDS) or
+// tile does.  Returns 0 (two launches), 1 (workgroups of 256 x 192 of both products, eight wavefronts, all of the LDS),
 // 2 (128 x 192 of both, four wavefronts: prompts of about 300 to 512 rows, where the 128 x 128 tile of a single product needs two
-// rounds of workgroups and this form one).  The model is choose_tile's: rounds of workgroups x outputs per workgroup / relative
+// rounds of workgroups and this form one) or 3 / 4 / 5 (32 / 64 / 128 rows x 64 columns of both: short prompts).  The model is choose_tile's: rounds of workgroups x outputs per workgroup / relative
 // throughput of a busy compute unit, with 1.23 x 1.18 measured for the 256-row form (7B and 13B shapes, 256 to 2048 prompt
 // rows: faster from 768 rows on except where the last round is nearly empty) and 0.87 for the 128-row form (7B shape: 3 - 4 % of
 // the time to the first token at 384 and 512 rows, slower at 256 and 640).
 static int choose_dual(const GemmParams &p) {
-    const char *env = getenv("RLLAMA_HIP_GEMM_DUAL"); // 0: never, 1 / 2: that form wherever the kernel can run (tests), unset: by shape; read at every call
+    const char *env = getenv("RLLAMA_HIP_GEMM_DUAL"); // 0: never, 1 ... 5: that form wherever the kernel can run (tests), unset: by shape; read at every call
     const int mode = env != nullptr ? atoi(env) : -1;
     if (mode == 0 || p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.k % 64 != 0) return 0;
     if ((p.ldc % 8) != 0 || (p.n % 8) != 0 || (reinterpret_cast<uintptr_t>(p.c) % 16) != 0) return 0;
-    if (mode == 1 || mode == 2) return mode;
+    if (mode >= 1 && mode <= 5) return mode;
+    // Up to 128 rows both products are bound by streaming their weights once, and one launch whose workgroups each take 64
+    // rows of w1 and the same 64 of w3 streams them at the rate of the single-row kernel (7B shape: 29.8 / 34.3 / 40.0 us at
+    // 16 / 48 / 128 rows against 41.7 / 49.1 / 60.3 us for two launches on 64 rows per workgroup; the single-row pair: 29.9).
+    // Beyond one round of such workgroups (65B shape: 344) only the 32-row form still gains (168 against 184 us).
+    if (p.m <= 128) {
+        const bool one_round = (p.n + 63) / 64 <= device_compute_units();
+        if (p.m <= 32) return 3;
+        if (one_round) return p.m <= 64 ? 4 : 5;
+    }
     double single = 0.0;
     const int tile = choose_tile(p, &single);
     if (tile < 0 || tile > 3 || choose_split_k(p, tile) != 1) return 0;
@@ -804,6 +815,9 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         const int dual = epilogue == kGemmEpiSiluGateF16 ? choose_dual(p_in) : 0;
         if (dual == 1) return launch_dma<kGemmEpiSiluGateF16, 4, 3, 64, 2, false, 2, true>(p_in, s); // 256 x 192 of both products, all of the LDS
         if (dual == 2) return launch_dma<kGemmEpiSiluGateF16, 2, 3, 64, 2, false, 2, true>(p_in, s); // 128 x 192 of both, four wavefronts
+        if (dual == 3) return launch_dma<kGemmEpiSiluGateF16, 1, 1, 64, 7, false, 1, true>(p_in, s); // 32 x 64 of both, two wavefronts
+        if (dual == 4) return launch_dma<kGemmEpiSiluGateF16, 1, 1, 64, 6, false, 2, true>(p_in, s); // 64 x 64 of both, two wavefronts
+        if (dual == 5) return launch_dma<kGemmEpiSiluGateF16, 2, 1, 64, 4, false, 2, true>(p_in, s); // 128 x 64 of both, four wavefronts
         return hipErrorInvalidValue;
     }
     if (epilogue == kGemmEpiSiluGateF16 && (p_in.gate == nullptr || p_in.batch != 1 || p_in.f32_operands)) return hipErrorInvalidValue;

@@ -174,7 +174,7 @@ def test_add_and_silu_mul(ctx):
         Tensor.from_numpy(ctx, ah).add(Tensor.from_numpy(ctx, bh))                                   # the residual stream is f32
 
 
-@pytest.mark.parametrize("n,m,k", [(300, 1000, 256), (256, 192, 64), (70, 520, 128), (513, 392, 192)])
+@pytest.mark.parametrize("n,m,k", [(300, 1000, 256), (256, 192, 64), (70, 520, 128), (513, 392, 192), (8, 264, 256), (100, 136, 192)])
 def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
     """FeedForward up to its gate for n rows (src/transformer.rs:551-565): the oracle's f16 matmul (src/tensor.rs:1282-1475,
     result rounded to f16), silu and hadamard product in f32, one rounding to f16.  The matrix cores add the k products in
@@ -192,7 +192,7 @@ def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
     X, W1, W3 = Tensor.from_numpy(ctx, x), Tensor.from_numpy(ctx, w1), Tensor.from_numpy(ctx, w3)
     got = {}
     os.environ["RLLAMA_HIP_GEMM_KGROUP"] = "0"  # the two-launch form on the kernel whose sum over k runs in the one-pass kernel's order
-    for mode in ("1", "2", "0"):
+    for mode in ("1", "2", "3", "4", "5", "0"):  # five shapes of the one-pass workgroup, two launches
         os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
         try:
             got[mode] = X.ffn_gate(W1, W3).to_numpy()
@@ -200,7 +200,8 @@ def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
             del os.environ["RLLAMA_HIP_GEMM_DUAL"]
     del os.environ["RLLAMA_HIP_GEMM_KGROUP"]
     assert np.array_equal(got["1"].view(np.uint16), got["0"].view(np.uint16))
-    assert np.array_equal(got["2"].view(np.uint16), got["0"].view(np.uint16))
+    for mode in ("2", "3", "4", "5"):
+        assert np.array_equal(got[mode].view(np.uint16), got["0"].view(np.uint16)), mode
     one = got["1"]
     step = np.spacing(np.maximum(np.abs(want), np.abs(one))).astype(f32)
     assert np.mean(one != want) < 2e-2 and np.all(np.abs(one.astype(f32) - want.astype(f32)) <= 2 * step)

@@ -321,14 +321,15 @@ def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n, monkeypatch):
     got = {}
     # (the two-launch form on the tile-splitting kernel, whose sum over k runs in the same order as the one-pass kernel's)
     monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", "0")
-    for mode in ("1", "2", "0"):  # workgroups of 256 rows (eight wavefronts), of 128 rows (four), two launches
+    # workgroups of 256 x 192 of both products (eight wavefronts), 128 x 192 (four), the short-prompt forms 32 / 64 / 128 x 64, two launches
+    for mode in ("1", "2", "3", "4", "5", "0"):
         os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
         try:
             gc = gm.make_caches()
             got[mode] = (gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc))
         finally:
             del os.environ["RLLAMA_HIP_GEMM_DUAL"]
-    for mode in ("1", "2"):
+    for mode in ("1", "2", "3", "4", "5"):
         assert np.array_equal(got[mode][0], got["0"][0]) and np.array_equal(got[mode][1], got["0"][1]), mode
     oc = om.make_caches()
     assert max_rel_err(got["1"][0], om.forward(toks[:n], 0, oc)) < TOL_F16
