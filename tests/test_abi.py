@@ -51,11 +51,11 @@ def test_rust_ffi_crate_matches_the_header():
         assert f"pub const {const}: c_int" in lib_rs
     for field in [f[0] for f in _lib.ModelParams._fields_] + [f[0] for f in _lib.SamplerParams._fields_]:
         assert f"pub {field}:" in lib_rs
-    # what INTEGRATION.md shows of the seam must exist in the crate
+    # every entry point that the integration guide at the repository root shows must exist in the crate
     doc = open(os.path.join(root, "INTEGRATION.md")).read()
     for name in set(re.findall(r"\b(rlh_[a-z0-9_]+)\b", doc)):
         assert name in decls or name in ("rlh_model_params", "rlh_sampler_params", "rlh_ctx", "rlh_model", "rlh_caches", "rlh_tensor", "rlh_event",
-                                         "rlh_tensor_kind", "rlh_status", "rlh_dtype"), f"INTEGRATION.md names {name}, which the header does not declare"
+                                         "rlh_tensor_kind", "rlh_status", "rlh_dtype"), f"the integration guide names {name}, which the header does not declare"
 
 
 def test_no_oracle_in_product():
