@@ -736,11 +736,17 @@ static int choose_split_k(const GemmParams &p, int tile) {
     // Worth it while the partial sums (pieces x m x n floats, written and read back) stay small beside the weights: products
     // whose tiles cover at most a quarter of the compute units (measured on the 7B shapes: wq|wk|wv / w1 / w3 on their 86 - 96
     // tiles are faster unsplit on the narrower 128 x 64 tile at any row count, wo / w2 on 32 tiles faster split)
-    const long max_blocks = n_cu / 4;
+    // -- and, with more than one row tile, products whose tiles cover at most half of them: a 128 x 128 tile takes as long
+    // with half the compute units idle as with all of them busy, so two pieces on twice the workgroups nearly halve the product
+    // (wo / w2 of the 7B shape at 320 / 384 / 512 rows: 10.0 / 10.7 / 11.1 -> 9.1 / 9.4 / 10.2 ms to the first token; three
+    // pieces measured the same as two; at 640 rows and more the tiles fill the part and a cut costs)
+    static const bool half_ok = !(getenv("RLLAMA_HIP_GEMM_SPLIT_HALF") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_SPLIT_HALF")) == 0);
+    const long max_blocks = p.m > 128 && half_ok ? n_cu / 2 : n_cu / 4;
     if (blocks > max_blocks && forced <= 1) return 1;
     // a single row tile runs its pieces on the 128 x 64 tile: twice the column tiles, half the pieces, half the partial sums
     const long tiles = p.m <= 128 ? (long)((p.n + 63) / 64) : blocks;
     long s = forced > 1 ? forced : (n_cu + tiles - 1) / tiles;
+    if (forced <= 1 && blocks > n_cu / 4) s = 2;
     if (s > k_tiles / 4) s = k_tiles / 4;                  // at least 4 K-tiles per piece
     const size_t per = (size_t)p.m * p.n * sizeof(float);
     if (per > 0 && (size_t)s * per > p.workspace_bytes) s = (long)(p.workspace_bytes / per);

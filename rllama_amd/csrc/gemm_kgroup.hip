@@ -15,7 +15,8 @@
 // order of g): deterministic, but not bit-identical to that kernel.
 //
 // Contract: GemmParams with batch 1, no K segments, no causal skipping, k % 64 == 0, lda / ldb % 8 == 0; epilogues
-// kGemmEpiF16 and kGemmEpiResAddF32.
+// kGemmEpiF16 and kGemmEpiResAddF32, and kGemmEpiF32 for the pieces of a product cut along K (batch = split_k K ranges as
+// grid.z, at least four K-tiles each, partial sums stride_c apart).
 #include "kernels.h"
 #include "device_utils.h"
 
@@ -65,7 +66,14 @@ __global__ __launch_bounds__(64 * kWM * kWN * kKG) void gemm_f16_kgroup_kernel(G
     }
     const int bm0 = by * kBM, bn0 = bx * kBN;
     const int M = p.m, N = p.n, K = p.k;
-    const int n_kt = K / kBK;
+    // split_k > 1: grid.z counts K ranges of one product -- range z takes K-tiles [z q + min(z, r), ...) of the K / 64 =
+    // split_k q + r tiles, one more for z < r -- and C item z (stride_c apart) gets its partial sum (kGemmEpiF32 only)
+    int n_kt = K / kBK, k_skip = 0;
+    if (p.split_k > 1) {
+        const int total = n_kt, q = total / p.split_k, r = total % p.split_k, z = (int)blockIdx.z;
+        n_kt = q + (z < r ? 1 : 0);
+        k_skip = (z * q + min(z, r)) * kBK;
+    }
 
     // ---- staging: a stage holds rows 0 .. kBM-1 of A then rows 0 .. kBN-1 of B, 128 bytes each, 16-byte chunk c of row r at
     //      chunk c ^ ((r / 2) % 8).  Addresses: a uniform base per matrix (tile origin + k) plus a 32-bit offset per load.
@@ -83,7 +91,7 @@ __global__ __launch_bounds__(64 * kWM * kWN * kKG) void gemm_f16_kgroup_kernel(G
         const int lc = l_pc ^ ((row / kSwzDiv) % kCpr);
         voff_b[i] = (unsigned)(((min(bn0 + row, N - 1) - bn0) * p.ldb + lc * 8) * 2);
     }
-    const half_t *s_a = p.a + (size_t)bm0 * p.lda, *s_b = p.b + (size_t)bn0 * p.ldb;
+    const half_t *s_a = p.a + (size_t)bm0 * p.lda + k_skip, *s_b = p.b + (size_t)bn0 * p.ldb + k_skip;
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_raw;
     int iss_k = 0;
     auto issue = [&](int kt) { // called for kt = 0, 1, 2, ... in this order
@@ -288,6 +296,7 @@ __global__ __launch_bounds__(64 * kWM * kWN * kKG) void gemm_f16_kgroup_kernel(G
                 if (r < M && c < N) {
                     const size_t off = (size_t)r * p.ldc + c;
                     if constexpr (kEpi == kGemmEpiF16) reinterpret_cast<half_t *>(p.c)[off] = (half_t)out[i][j][v];
+                    else if constexpr (kEpi == kGemmEpiF32) reinterpret_cast<float *>(p.c)[(size_t)blockIdx.z * p.stride_c + off] = out[i][j][v]; // a piece's partial sum
                     else reinterpret_cast<float *>(p.c)[off] = early[i][j][v] + f16r(out[i][j][v]); // transformer.rs:442 / :445 on the f16-rounded product
                 }
             }
@@ -301,8 +310,10 @@ bool gemm_f16_kgroup_supported(const GemmParams &p, int epilogue, int tile) {
     // and 112.4 against 111 us with RoPE and the cache write in the epilogue: the cycles fall as the LDS bytes do, the clock
     // falls with them (power), and the exchange of the partial sums is added.  Not wired in.)
     if (tile != 0 && tile != 4) return false;
-    if (epilogue != kGemmEpiF16 && epilogue != kGemmEpiResAddF32) return false;
-    if (p.f32_operands || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.b2 != nullptr || p.split_k > 1 || p.accumulate) return false;
+    if (epilogue != kGemmEpiF16 && epilogue != kGemmEpiResAddF32 && epilogue != kGemmEpiF32) return false;
+    // (fp32 store: the pieces of a product cut along K, as the launcher of gemm_dma.hip sets them up -- batch = split_k pieces)
+    if (epilogue == kGemmEpiF32 ? (p.split_k < 2 || p.batch != p.split_k || p.k / 64 / p.split_k < 4) : (p.split_k > 1 || p.batch != 1)) return false;
+    if (p.f32_operands || p.k_seg != 0 || p.causal != 0 || p.b2 != nullptr || p.accumulate) return false;
     if (p.m <= 0 || p.n <= 0 || p.k < 64 || p.k % 64 != 0 || p.lda % 8 != 0 || p.ldb % 8 != 0) return false;
     if (epilogue == kGemmEpiResAddF32 && p.residual == nullptr) return false;
     return true;
@@ -316,7 +327,7 @@ static hipError_t launch_kgroup(const GemmParams &p, hipStream_t s) {
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f16_kgroup_kernel<kEpi, kWM, kWN, kKG, kIT, kNT, kStages>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) return attr;
-    const dim3 grid((p.n + bn - 1) / bn, (p.m + bm - 1) / bm, 1);
+    const dim3 grid((p.n + bn - 1) / bn, (p.m + bm - 1) / bm, p.split_k > 1 ? p.split_k : 1);
     hipLaunchKernelGGL((gemm_f16_kgroup_kernel<kEpi, kWM, kWN, kKG, kIT, kNT, kStages>), grid, dim3(64 * kWM * kWN * kKG), lds, s, p);
     return hipGetLastError();
 }
@@ -327,6 +338,7 @@ hipError_t launch_gemm_f16_kgroup(const GemmParams &p, int epilogue, int tile, h
     // four (the whole tile per wavefront -- 256 accumulator registers -- does not survive hipcc's register allocation); four
     // stages of 32 KB
     if (epilogue == kGemmEpiF16) return launch_kgroup<kGemmEpiF16, 1, 2, 4, 4, 2, 4>(p, s);
+    if (epilogue == kGemmEpiF32) return launch_kgroup<kGemmEpiF32, 1, 2, 4, 4, 2, 4>(p, s);
     return launch_kgroup<kGemmEpiResAddF32, 1, 2, 4, 4, 2, 4>(p, s);
 }
 
