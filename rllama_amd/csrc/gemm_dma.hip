@@ -792,7 +792,9 @@ static int choose_dual(const GemmParams &p) {
     const double dual256 = (double)((blocks256 + n_cu - 1) / n_cu) * 2.0 * 256 * 192 / (1.23 * 1.18);
     const double dual128 = (double)((blocks128 + n_cu - 1) / n_cu) * 2.0 * 128 * 192 / 0.87;
     const double best = dual256 <= dual128 ? dual256 : dual128;
-    if (best >= 2.0 * single) return 0;
+    // (10 % in favour of the pass: with three row tiles -- 520 to 768 rows -- it runs on 174 workgroups at a higher clock than
+    // the model's unit assumes, 145.6 us at the 7B shape against 84.5 + 77.3 us for two launches of 128 x 128 tiles in two rounds)
+    if (best >= 2.0 * single * 1.1) return 0;
     return dual256 <= dual128 ? 1 : 2;
 }
 
