@@ -20,6 +20,9 @@
 // that is the only numerical difference.
 #include "gemv_device.h"
 
+#include <cstdlib>
+#include <type_traits>
+
 namespace rlh {
 
 size_t gemv_lds_bytes(int k, int w_is_f16, int x_f16) {
@@ -27,7 +30,7 @@ size_t gemv_lds_bytes(int k, int w_is_f16, int x_f16) {
     return (size_t)gemv_iters(k, vec) * kWave * vec * (x_f16 ? 2 : 4);
 }
 
-template <typename WT, typename XT, int kEpi, bool kStream>
+template <typename WT, typename XT, int kEpi, bool kStream, int kBurst = kGemvBurst>
 __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     extern __shared__ uint4_t smem_raw[];
     __shared__ float red[16];
@@ -35,8 +38,8 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     // (measured: issuing the first burst behind the prologue's loads is worth 1 % on the w1|w3 product, nothing or a loss on
     // the others, so only that instantiation does it)
     constexpr int kPre = (RLH_GEMV_PRELOAD && kEpi == kEpiSilu) ? kPreSelf : kPreNone;
-    uint4_t wpre[1][kGemvBurst];
-    gemv_body<WT, XT, kEpi, kStream, false, kPre>(p, smem_raw, red, rope_f, wpre, 0u);
+    uint4_t wpre[1][kBurst];
+    gemv_body<WT, XT, kEpi, kStream, false, kPre, false, 1, kBurst>(p, smem_raw, red, rope_f, wpre, 0u);
 }
 
 template <typename WT, typename XT, int kEpi>
@@ -54,6 +57,31 @@ static hipError_t launch_gemv_t(GemvParams p, hipStream_t s) {
         hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemvThreads), lds, s, p);
         return hipGetLastError();
     };
+    // f16 weights: a burst length that divides the row into whole bursts, where one of these does (pieces of 512 halves per row,
+    // LLaMA shapes: 8 / 10 / 16 for dim 4096 / 5120 / 8192, 21.5 -> 22 / 27 / 35 for ffn 11008 / 13824 / 17920; 13 and 43 --
+    // dim 6656, ffn 22016 -- have no divisor here and keep the default with its partial last burst).  Same order of additions
+    // per lane whatever the burst length, so the same bits.  Measured: w2 of the 7B shape 18.8 -> 17.3 us, wo of the 13B shape
+    // 12.2 -> 11.1 us, w2 of the 13B shape 25.7 -> 25.4 us.
+    if constexpr (std::is_same<WT, half_t>::value) {
+        constexpr int mr = GemvShape<WT, kEpi>::kMats * GemvShape<WT, kEpi>::kRows;
+        static const bool fixed = getenv("RLLAMA_HIP_GEMV_BURST") != nullptr && atoi(getenv("RLLAMA_HIP_GEMV_BURST")) == 0; // 0: always the default length
+        const int pieces = gemv_iters(p.k, WVec<WT>::kVec);
+        auto pick = [&](auto burst) -> hipError_t {
+            constexpr int kB = decltype(burst)::value;
+            if (p.stream_weights) return launch(gemv_kernel<WT, XT, kEpi, true, kB>);
+            return launch(gemv_kernel<WT, XT, kEpi, false, kB>);
+        };
+        if (!fixed && pieces % (kGemvBurst / mr) != 0) {
+            // (one matrix, one row per unit only: the 13B shape's wq|wk|wv and w1|w3, 10 pieces per row as 5 + 5 instead of
+            // 4 + 4 + 2 for each of two rows, measured 30.1 against 29.2 us and 46.6 against 46.4 us)
+            if constexpr (mr == 1) {
+                if (pieces % 9 == 0) return pick(std::integral_constant<int, 9>{});
+                if (pieces % 10 == 0) return pick(std::integral_constant<int, 10>{});
+                if (pieces % 11 == 0) return pick(std::integral_constant<int, 11>{});
+                if (pieces % 7 == 0) return pick(std::integral_constant<int, 7>{});
+            }
+        }
+    }
     if (p.stream_weights) return launch(gemv_kernel<WT, XT, kEpi, true>);
     return launch(gemv_kernel<WT, XT, kEpi, false>);
 }

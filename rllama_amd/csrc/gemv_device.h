@@ -154,12 +154,15 @@ enum GemvPreload {
     kPreGiven = 2   // issued by the caller before this phase began (the fused kernel issues it before the barrier it waits at)
 };
 
-template <typename WT, int kEpi>
+// kBurst: 16-byte loads per lane and burst.  Rows that divide into whole bursts stream about 1 us faster per product than rows
+// whose last burst is a partial one (7B shape, k = 11008 = 21.5 pieces: 18.4 us with bursts of 8 + 8 + 6, 17.3 us with 11 + 11),
+// so the launcher picks a burst length that divides the row where one of the instantiated lengths does.
+template <typename WT, int kEpi, int kBurst = kGemvBurst>
 struct GemvShape {
     static constexpr int kVec = WVec<WT>::kVec;
     static constexpr int kMats = (kEpi == kEpiSilu) ? 2 : 1;    // w1 and w3 share x and the epilogue
     static constexpr int kRows = (kEpi == kEpiRopeKv) ? 2 : 1;  // a RoPE pair (2j, 2j+1) is produced by one wave
-    static constexpr int kU = kGemvBurst / (kMats * kRows);     // pieces of one row per burst
+    static constexpr int kU = kBurst / (kMats * kRows);         // pieces of one row per burst
     static constexpr int kPiece = kWave * kVec;                  // elements one wave-wide load covers
 };
 
@@ -167,9 +170,9 @@ struct GemvShape {
 // unit the pieces 0, kU, 2 kU, ...  This issues the loads of the first kD of them into wpre and returns a mask of those it
 // issued (bit d: burst d is in wpre[d]); a burst that does not exist or is not a full one (the ragged end of a row) is left
 // to the main loop.  The loads do not depend on x.
-template <typename WT, int kEpi, bool kStream, int kD>
-__device__ __forceinline__ unsigned gemv_issue_bursts(const GemvParams &p, uint4_t (&wpre)[kD][kGemvBurst]) {
-    using S = GemvShape<WT, kEpi>;
+template <typename WT, int kEpi, bool kStream, int kD, int kBurst = kGemvBurst>
+__device__ __forceinline__ unsigned gemv_issue_bursts(const GemvParams &p, uint4_t (&wpre)[kD][kBurst]) {
+    using S = GemvShape<WT, kEpi, kBurst>;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int K = p.k;
@@ -205,10 +208,10 @@ __device__ __forceinline__ unsigned gemv_issue_bursts(const GemvParams &p, uint4
 // One GEMV over the whole grid: prologue (x staged in LDS), main loop, epilogue.  `smem_raw` is the block's dynamic LDS
 // (gemv_lds_bytes); `red` 16 floats and `rope_f` 64 float2 of static LDS.  kDev: x / x_add are read and y / x_out written at
 // device scope (see above).  With kPre == kPreGiven, wpre holds the first kD bursts the caller issued and pre_mask says which.
-template <typename WT, typename XT, int kEpi, bool kStream, bool kDev, int kPre, bool kDevLoad = false, int kD = 1>
-__device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f, uint4_t (&wpre)[kD][kGemvBurst],
+template <typename WT, typename XT, int kEpi, bool kStream, bool kDev, int kPre, bool kDevLoad = false, int kD = 1, int kBurst = kGemvBurst>
+__device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f, uint4_t (&wpre)[kD][kBurst],
                                           unsigned pre_mask) {
-    using S = GemvShape<WT, kEpi>;
+    using S = GemvShape<WT, kEpi, kBurst>;
     constexpr int kVec = S::kVec, kMats = S::kMats, kRows = S::kRows, kU = S::kU, kPiece = S::kPiece;
     XT *xs = reinterpret_cast<XT *>(smem_raw);
 
@@ -225,7 +228,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     if constexpr (kMats == 2) wmat[1] = reinterpret_cast<const WT *>(p.w_b);
     const int unit_first = blockIdx.x * kGemvWaves + wave;
     auto preload = [&]() {
-        if constexpr (kPre == kPreSelf) pre_mask = gemv_issue_bursts<WT, kEpi, kStream, kD>(p, wpre);
+        if constexpr (kPre == kPreSelf) pre_mask = gemv_issue_bursts<WT, kEpi, kStream, kD, kBurst>(p, wpre);
         __builtin_amdgcn_sched_barrier(0);
     };
     if constexpr (kPre == kPreNone) pre_mask = 0;
@@ -357,6 +360,17 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
 #pragma unroll
                     for (int r = 0; r < kRows; r++)
                         wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + (size_t)(c + u) * kPiece + lane * kVec);
+        } else if (c + kU <= pieces) {
+            // the row ends with this burst in a partial piece: every piece exists, lanes past the end of the row are clamped
+            // to valid weights (they meet zeros of the padded x)
+#pragma unroll
+            for (int u = 0; u < kU; u++) {
+                const int kk = min((c + u) * kPiece + lane * kVec, K - kVec);
+#pragma unroll
+                for (int m = 0; m < kMats; m++)
+#pragma unroll
+                    for (int r = 0; r < kRows; r++) wv[u][m][r] = load16<kStream>(wmat[m] + (size_t)(row0 + r) * K + kk);
+            }
         } else {
             // tail burst: pieces past the end are skipped, the partial last piece is clamped to valid
             // weights (they meet zeros of the padded x)
