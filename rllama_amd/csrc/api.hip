@@ -777,6 +777,7 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
         GemvParams p;
         int epi = kEpiStore;
         build_gemv_step(m, c, l, which, first_layer, &p, &epi);
+        if (which == kStepQkv && !m->capturing) p.pos1_host = T_host; // (a captured step is replayed at later positions: it reads the device state)
         HIP_TRY(launch_gemv(p, epi, st));
         return RLH_OK;
     }

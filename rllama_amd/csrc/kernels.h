@@ -41,6 +41,7 @@ struct GemvParams {
     int rows_per_wave;        // set by launch_gemv
     // kEpiRopeKv only
     const DecodeState *state;
+    int pos1_host;            // position + 1 where the host knows it (spares the kernel a dependent load), 0: read state->pos
     const float2 *freqs;      // [max_seq_len x head_dim/2] (cos, sin) as f32
     void *cache_k;            // this layer's K cache [n_heads x max_seq_len x head_dim]
     void *cache_v;
