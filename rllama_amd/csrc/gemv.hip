@@ -3,8 +3,9 @@
 // One token step reads every weight byte exactly once, so this kernel is bound by HBM bandwidth and is
 // built as a streaming reader:
 //   * a wavefront produces one output row at a time with 16-byte loads per lane (one load instruction
-//     covers 1 KiB of the row), issued in bursts of 8 independent loads whose addresses differ by
-//     compile-time offsets, so the per-load instruction overhead is one VMEM instruction;
+//     covers 1 KiB of the row), issued in bursts of 8 independent loads (7 to 11 where that divides the row
+//     and 8 does not) whose addresses differ by compile-time offsets, so the per-load instruction overhead
+//     is one VMEM instruction;
 //   * rows are interleaved over all wavefronts of the grid (wave w takes rows w, w + W, ...), so that at
 //     any moment the grid reads one dense window of the matrix, and the launch is sized so that all
 //     wavefronts are resident at once (about 8 per CU);
