@@ -65,7 +65,8 @@ static hipError_t launch_gemv_t(GemvParams p, hipStream_t s) {
     // 12.2 -> 11.1 us, w2 of the 13B shape 25.7 -> 25.4 us.
     if constexpr (std::is_same<WT, half_t>::value) {
         constexpr int mr = GemvShape<WT, kEpi>::kMats * GemvShape<WT, kEpi>::kRows;
-        static const bool fixed = getenv("RLLAMA_HIP_GEMV_BURST") != nullptr && atoi(getenv("RLLAMA_HIP_GEMV_BURST")) == 0; // 0: always the default length
+        const char *env = getenv("RLLAMA_HIP_GEMV_BURST"); // 0: always the default length; read at every call
+        const bool fixed = env != nullptr && atoi(env) == 0;
         const int pieces = gemv_iters(p.k, WVec<WT>::kVec);
         auto pick = [&](auto burst) -> hipError_t {
             constexpr int kB = decltype(burst)::value;

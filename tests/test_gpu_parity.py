@@ -83,6 +83,29 @@ def test_gemv_f16_weights(ctx, m_rows, k):
     assert np.allclose(got_head, exact_head, rtol=1e-5, atol=1e-5 * np.abs(exact_head).max())
 
 
+@pytest.mark.parametrize("m_rows,k,burst", [(300, 11008, 11), (130, 5376, 11), (64, 4608, 9), (2100, 13824, 9), (77, 5120, 10), (40, 3584, 7), (9, 6656, 8)])
+def test_gemv_burst_length_follows_the_row(ctx, m_rows, k, burst, monkeypatch):
+    """The single-row product issues its loads in bursts of 7, 9, 10 or 11 per lane where that divides the row's pieces of 512
+    halves and 8 does not (a row that ends inside a piece counts as whole pieces: 11008 -> 22, 5376 -> 11); the last case has
+    13 pieces and keeps 8 with a partial last burst.  Every lane still adds its products in the order of the pieces, so the
+    bits are those of the fixed burst length; and against the oracle (tensor.rs:1476-1666)."""
+    assert -(-k // 512) % burst == 0 or burst == 8
+    rng = np.random.default_rng(m_rows + k)
+    wh = oracle.f32_to_f16_bits((rng.standard_normal((m_rows, k)) * 0.05).astype(f32))
+    x = rng.standard_normal((1, k)).astype(f32)
+    xh = oracle.f32_to_f16_bits(x)
+    W, X = Tensor.from_numpy(ctx, wh), Tensor.from_numpy(ctx, x)
+    got = W.gemv(X, round_x=True, round_y=True).to_numpy()[0]
+    got32 = W.gemv(X, round_x=False, round_y=False).to_numpy()[0]
+    monkeypatch.setenv("RLLAMA_HIP_GEMV_BURST", "0")
+    assert np.array_equal(got, W.gemv(X, round_x=True, round_y=True).to_numpy()[0])
+    assert np.array_equal(got32, W.gemv(X, round_x=False, round_y=False).to_numpy()[0])
+    want = oracle.f16_bits_to_f32(oracle.matmul_transposed_f16(xh, wh))[0]
+    mag = np.abs(oracle.f16_bits_to_f32(xh).astype(np.float64))[0] @ np.abs(oracle.f16_bits_to_f32(wh).astype(np.float64)).T
+    close_f16(got, want, mag, "gemv f16, burst length by row")
+    assert np.mean(got != want) < 0.02
+
+
 @pytest.mark.parametrize("m_rows,k", [(5, 4), (64, 512), (1000, 1000), (4096, 4096)])
 def test_gemv_f32_weights(ctx, m_rows, k):
     rng = np.random.default_rng(m_rows * 17 + k)
