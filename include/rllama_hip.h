@@ -226,7 +226,8 @@ int  rlh_silu_inplace(rlh_tensor *t);                                           
 /* OpenCLTensor::matrix_mul_inplace_transposed(self, src, other) (:301-405): dst[r, c] = sum_k src[r, k] * other[c, k].
  * src [n x k], other [m x k], dst [n x m].  f16 operands give an f16-rounded dst (as src/tensor.rs:1623-1643);
  * f32 operands give f32.  src and other must share a dtype; dst has it too.  n == 1 takes the GEMV kernel,
- * n > 1 the MFMA GEMM (f16) or the tiled fp32 kernel. */
+ * n > 1 the MFMA GEMM (f16) or the tiled fp32 kernel.  The first call with n > 1 on a context allocates a 64 MiB workspace
+ * that stays with the context (partial sums of products cut along K, as inside the forward; rlh_ffn_gate shares it). */
 int  rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tensor *src, const rlh_tensor *other);
 /* Decode GEMV with the rounding switches of the fused path: y[c] = sum_k x[k] * W[c, k]; x f32 [1 x k]
  * (rounded to f16 first if round_x), W f16 or f32 [m x k], y f32 [1 x m] (rounded to f16 precision if round_y). */
