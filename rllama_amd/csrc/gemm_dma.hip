@@ -768,7 +768,11 @@ static hipError_t launch_split_finish(const GemmParams &p, int splits, hipStream
 // throughput of a busy compute unit, with 1.23 x 1.18 measured for the 256-row form (7B and 13B shapes, 256 to 2048 prompt
 // rows: faster from 768 rows on except where the last round is nearly empty) and 0.87 for the 128-row form (7B shape: 3 - 4 % of
 // the time to the first token at 384 and 512 rows, slower at 256 and 640).
-static int choose_dual(const GemmParams &p) {
+// *cut_cols (optional) receives a number of columns n1 > 0 when the 256-row form should run on the first n1 columns only
+// and the remaining columns as two launches: where the workgroups of the pass make whole rounds and a bit (13B shape, 2048
+// rows: 576 = 2.25 rounds of 256), the bit costs a whole round, and as two small products it costs a fraction of one.
+static int choose_dual(const GemmParams &p, int *cut_cols = nullptr) {
+    if (cut_cols != nullptr) *cut_cols = 0;
     const char *env = getenv("RLLAMA_HIP_GEMM_DUAL"); // 0: never, 1 ... 5: that form wherever the kernel can run (tests), unset: by shape; read at every call
     const int mode = env != nullptr ? atoi(env) : -1;
     if (mode == 0 || p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.k % 64 != 0) return 0;
@@ -789,16 +793,40 @@ static int choose_dual(const GemmParams &p) {
     const int n_cu = device_compute_units();
     const long cols = (p.n + 191) / 192;
     const long blocks256 = cols * ((p.m + 255) / 256), blocks128 = cols * ((p.m + 127) / 128);
-    const double dual256 = (double)((blocks256 + n_cu - 1) / n_cu) * 2.0 * 256 * 192 / (1.23 * 1.18);
+    const double unit256 = 2.0 * 256 * 192 / (1.23 * 1.18);
+    double dual256 = (double)((blocks256 + n_cu - 1) / n_cu) * unit256;
     const double dual128 = (double)((blocks128 + n_cu - 1) / n_cu) * 2.0 * 128 * 192 / 0.87;
+    // the 256-row form on the columns that make whole rounds, the rest (at most a quarter of a round of its workgroups) as two
+    // launches; 3 us per additional launch in the model's unit (6.2e-7 us x K each)
+    static const bool cut_ok = !(getenv("RLLAMA_HIP_GEMM_DUAL_CUT") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_DUAL_CUT")) == 0);
+    const long rows256 = (p.m + 255) / 256, full = blocks256 / n_cu, cols_main = full * n_cu / rows256;
+    int n1 = 0;
+    // (from two whole rounds on: with one, 7B shape 1280 rows and 13B shape 1024 rows, the cut measured 3 % slower than without)
+    if (cut_ok && cut_cols != nullptr && full >= 2 && cols_main >= 1 && cols_main < cols && (cols - cols_main) * rows256 * 4 <= n_cu) {
+        GemmParams r = p;
+        r.n = p.n - (int)cols_main * 192;
+        r.b2 = nullptr;
+        double rest = 0.0;
+        const int rt = choose_tile(r, &rest);
+        const double launch = 3.0 / (6.2e-7 * p.k);
+        const double with_cut = (double)full * unit256 + 2.0 * rest + 2.0 * launch;
+        if (rt >= 0 && with_cut < dual256) {
+            dual256 = with_cut;
+            n1 = (int)cols_main * 192;
+        }
+    }
     const double best = dual256 <= dual128 ? dual256 : dual128;
     // (10 % in favour of the pass: with three row tiles -- 520 to 768 rows -- it runs on 174 workgroups at a higher clock than
     // the model's unit assumes, 145.6 us at the 7B shape against 84.5 + 77.3 us for two launches of 128 x 128 tiles in two rounds)
     if (best >= 2.0 * single * 1.1) return 0;
+    if (dual256 <= dual128 && cut_cols != nullptr) *cut_cols = n1;
     return dual256 <= dual128 ? 1 : 2;
 }
 
-bool gemm_f16_dual_gate_supported(const GemmParams &p) { return choose_dual(p) != 0; }
+bool gemm_f16_dual_gate_supported(const GemmParams &p) {
+    int n1 = 0;
+    return choose_dual(p, &n1) != 0;
+}
 
 // The RoPE epilogue needs whole 16-byte pieces everywhere and an unsplit product (a product cut along K has its epilogue in
 // the kernel that adds the partial sums; the caller then stores the product and runs the separate kernel).
@@ -820,7 +848,25 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
     if (epilogue == kGemmEpiResAddF32 && (p_in.residual == nullptr || p_in.batch != 1)) return hipErrorInvalidValue;
     if (epilogue == kGemmEpiRopeQkv && !gemm_f16_rope_supported(p_in)) return hipErrorInvalidValue;
     if (p_in.b2 != nullptr) {
-        const int dual = epilogue == kGemmEpiSiluGateF16 ? choose_dual(p_in) : 0;
+        int n1 = 0;
+        const int dual = epilogue == kGemmEpiSiluGateF16 ? choose_dual(p_in, &n1) : 0;
+        if (dual == 1 && n1 > 0) {
+            GemmParams left = p_in, right = p_in;
+            left.n = n1;
+            hipError_t e = launch_dma<kGemmEpiSiluGateF16, 4, 3, 64, 2, false, 2, true>(left, s);
+            if (e != hipSuccess) return e;
+            // the other columns: w1's product into C, then w3's with C as its gate (every element of the gate is read by the
+            // lane that overwrites it)
+            right.n = p_in.n - n1;
+            right.b = p_in.b + (size_t)n1 * p_in.ldb;
+            right.b2 = nullptr;
+            right.c = reinterpret_cast<half_t *>(p_in.c) + n1;
+            e = launch_gemm_f16_dma(right, kGemmEpiF16, s);
+            if (e != hipSuccess) return e;
+            right.b = p_in.b2 + (size_t)n1 * p_in.ldb;
+            right.gate = reinterpret_cast<const half_t *>(right.c);
+            return launch_gemm_f16_dma(right, kGemmEpiSiluGateF16, s);
+        }
         if (dual == 1) return launch_dma<kGemmEpiSiluGateF16, 4, 3, 64, 2, false, 2, true>(p_in, s); // 256 x 192 of both products, all of the LDS
         if (dual == 2) return launch_dma<kGemmEpiSiluGateF16, 2, 3, 64, 2, false, 2, true>(p_in, s); // 128 x 192 of both, four wavefronts
         if (dual == 3) return launch_dma<kGemmEpiSiluGateF16, 1, 1, 64, 7, false, 1, true>(p_in, s); // 32 x 64 of both, two wavefronts

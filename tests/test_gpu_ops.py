@@ -211,6 +211,37 @@ def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
         Tensor.from_numpy(ctx, x.astype(f32)).ffn_gate(W1, W3)                                       # f16 mode only
 
 
+def test_ffn_gate_whole_rounds_in_one_pass_and_the_rest_in_two_launches(ctx, monkeypatch):
+    """2048 rows x 13824 columns are 576 workgroups of the one-pass form, 2.25 rounds of the 256 compute units: the pass takes
+    the 12288 columns that make two whole rounds and the last 1536 go through w1's product and w3's with the gate epilogue
+    (src/transformer.rs:551-565 either way).  Against the two-launch form over all columns (a few f16 steps apart on few
+    elements: the remaining columns add their k products in another order, and a gate or product that lands on the neighbouring
+    f16 value moves the result by up to its own relative step each) and, on a sample, against float64."""
+    import os
+    n, m, k = 2048, 13824, 1024
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((n, k)) * 0.5).astype(np.float16)
+    w1 = (rng.standard_normal((m, k)) * 0.05).astype(np.float16)
+    w3 = (rng.standard_normal((m, k)) * 0.05).astype(np.float16)
+    X, W1, W3 = Tensor.from_numpy(ctx, x), Tensor.from_numpy(ctx, w1), Tensor.from_numpy(ctx, w3)
+    monkeypatch.delenv("RLLAMA_HIP_GEMM_DUAL", raising=False)
+    got = X.ffn_gate(W1, W3).to_numpy()
+    monkeypatch.setenv("RLLAMA_HIP_GEMM_DUAL", "0")
+    two = X.ffn_gate(W1, W3).to_numpy()
+    monkeypatch.delenv("RLLAMA_HIP_GEMM_DUAL")
+    step = np.spacing(np.maximum(np.abs(got), np.abs(two))).astype(f32)
+    assert np.array_equal(got[:, :12288], two[:, :12288])   # the pass: the two-launch form's order of additions
+    assert np.mean(got[:, 12288:] != two[:, 12288:]) < 5e-3 and np.all(np.abs(got.astype(f32) - two.astype(f32)) <= 8 * step)
+    rows = rng.integers(0, n, 600)
+    cols = np.concatenate([rng.integers(0, 12288, 300), rng.integers(12288, m, 300)])  # both sides of the cut
+    xs, a, b = x[rows].astype(np.float64), w1[cols].astype(np.float64), w3[cols].astype(np.float64)
+    g = np.einsum("ik,ik->i", xs, a).astype(np.float16).astype(np.float64)
+    u = np.einsum("ik,ik->i", xs, b).astype(np.float16).astype(np.float64)
+    want = (g / (1.0 + np.exp(-g)) * u)
+    have = got[rows, cols].astype(np.float64)
+    assert np.all(np.abs(have - want) <= 4e-3 * np.abs(want) + 1e-4), float(np.max(np.abs(have - want)))
+
+
 @pytest.mark.parametrize("parts", [2, 4])
 @pytest.mark.parametrize("hd,H,n", [(128, 2, 200), (64, 3, 65), (128, 1, 64), (64, 2, 1), (128, 2, 333)])
 def test_attn_prefill_against_the_reference_ops(ctx, hd, H, n, parts, monkeypatch):
