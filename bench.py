@@ -154,6 +154,47 @@ def measure_prefill(ra, ctx, model, prompt, reps, dim, n_layers, ffn, vocab):
     return wall_ms, ev_ms, tflops, gemm_us, gemm_tflops, gemm_flops, flops_total
 
 
+def other_config_block(ra, ctx, name, warmup=8, kernel_iters=160):
+    """One of the other decode configurations of the benchmark definition, measured like the headline one: its own model
+    (random-init, seed 0), its prompt through the matrix-core path, then its K greedy decode steps timed between two syncs;
+    the token-step kernels timed one by one at the mean sequence length of those steps."""
+    dim, n_layers, n_heads, ffn, vocab, n_prompt, K = CONFIGS[name]
+    max_seq = n_prompt + max(K, warmup) + 1
+    model = ra.Transformer(ctx, dim, n_layers, n_heads, ffn, vocab, max_seq, 1e-6, ra.DataSettings(ctx).force_f16())
+    model.fill_synthetic(seed=0, std=0.02)
+    prompt = ra.synth_tokens(0, n_prompt, 3, vocab)
+    cw = model.make_caches()
+    model.generate_greedy(prompt, 1, cw)                     # sizes the work buffers
+    model.decode_greedy(warmup, cw)
+    cw.free()
+    caches = model.make_caches()
+    ctx.sync()
+    t0 = time.perf_counter()
+    _, ms_prompt, _ = model.generate_greedy(prompt, 1, caches)
+    ctx.sync()
+    prompt_wall = 1e3 * (time.perf_counter() - t0)
+    t0 = time.perf_counter()
+    _, ms_events = model.decode_greedy(K, caches)
+    ctx.sync()
+    ms = 1e3 * (time.perf_counter() - t0) / K
+    mean_bytes = float(np.mean([model.decode_bytes(n_prompt + i + 1) for i in range(K)]))
+    T_mid = n_prompt + K // 2
+    kernels = {}
+    for which, kname in enumerate(ra.Transformer.STEP_KERNELS):
+        us, nbytes = model.time_kernel(which, T_mid, kernel_iters if which != 5 else max(20, kernel_iters // 8), caches)
+        kernels[kname] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3)}
+    caches.free()
+    model.free()
+    return {
+        "workload": f"{name}: dim {dim}, {n_layers} layers, {n_heads} heads, ffn {ffn}, vocab {vocab}; {n_prompt} prompt ids then {K} greedy decode tokens, batch 1",
+        "ms_per_token": round(ms, 4), "ms_per_token_hip_events": round(ms_events / K, 4), "tokens_per_s": round(1e3 / ms, 2),
+        "algorithmic_bytes_per_token": int(mean_bytes), "hbm_GBps_end_to_end": round(mean_bytes / (ms * 1e-3) / 1e9, 1),
+        "hbm_frac_end_to_end": round(mean_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "ms_prompt_pass": round(ms_prompt, 2), "ms_prompt_pass_wall": round(prompt_wall, 2), "prompt_tokens": n_prompt,
+        "kernels_at_T": T_mid, "kernels": kernels,
+    }
+
+
 def bench_layer_split(args, ra, ctx, info) -> int:
     """The device's share of a model split by percentage_to_gpu: one prompt call, then K single-token calls of
     rlh_forward_layers, each taking the stream from host memory and returning it there (the hand-off the reference makes at
@@ -212,6 +253,7 @@ def main() -> int:
     ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill-block", action="store_true", help="c1: skip the 1024-token prefill measurement (prefill_c3)")
+    ap.add_argument("--no-other-configs", action="store_true", help="c1: skip the 13B (c2) and 65B (c4) decode measurements (other_configs)")
     ap.add_argument("--kernel-iters", type=int, default=320)
     ap.add_argument("--kernels-only", action="store_true",
                     help="skip the token loop and the CPU baseline: only the per-kernel timing loops (short runs for "
@@ -298,9 +340,6 @@ def main() -> int:
                 continue
             us, nbytes = model.time_kernel(which, T_mid, args.kernel_iters, caches)
             out["kernels"][name] = {"us": round(us, 2), "bytes": nbytes}
-        if not args.kernel or args.kernel == "fused_layer":
-            us, nbytes = model.time_kernel(ra.Transformer.FUSED_LAYER_KERNEL, T_mid, args.kernel_iters, caches)
-            out["kernels"]["fused_layer"] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
         print(json.dumps(out))
         return 0
 
@@ -401,6 +440,15 @@ def main() -> int:
         out["cpu_baseline"] = None
     caches.free()
     model.free()
+    if args.config == "c1" and not args.no_other_configs:
+        # the other two decode configurations of the benchmark definition, each on its own model (the 7B one is freed first:
+        # the 65B weights alone are 130 GB)
+        out["other_configs"] = {}
+        for name in ("c2", "c4"):
+            try:
+                out["other_configs"][name] = other_config_block(ra, ctx, name)
+            except ra.RllamaHipError as e:   # e.g. a smaller part without room for the 65B shape: say so, keep the headline line
+                out["other_configs"][name] = {"error": str(e)}
     ctx.close()
     print(json.dumps(out))
     return 0

@@ -75,6 +75,12 @@ void rlh_shutdown(rlh_ctx *ctx);
  * when all work queued on the context has completed. */
 int  rlh_sync(rlh_ctx *ctx);
 const char *rlh_last_error(void);
+/* The library's switches (no reference counterpart: the reference has compile-time features only, Cargo.toml:42-44).
+ * rlh_init reads RLLAMA_HIP_<NAME> from the environment once per context; nothing reads the environment afterwards, and
+ * this call is the only other way to change a switch: name = NAME without the prefix ("GEMM_DUAL", "ATTN_MERGE", ...),
+ * value = what the variable would hold, NULL = back to the default.  Waits for the context's queued work first; applies to
+ * every later call on the context.  Unknown names and unusable values are RLH_ERR_INVALID. */
+int  rlh_set_option(rlh_ctx *ctx, const char *name, const char *value);
 /* Device facts for reports: name (<= cap bytes incl. NUL), compute units, total HBM bytes. */
 int  rlh_device_info(rlh_ctx *ctx, char *name, int cap, int *compute_units, uint64_t *hbm_bytes);
 
@@ -293,8 +299,7 @@ int  rlh_argmax_greedy(const rlh_tensor *logits, float temperature, int32_t *tok
  * ---------------------------------------------------------------------------------------------- */
 /* One kernel of the token step, cycling through the layers so that every launch streams different weights.
  * which: 0 = attention_norm + wq|wk|wv + RoPE + cache write, 1 = single-query attention at sequence length T,
- * 2 = wo + residual, 3 = ffn_norm + w1|w3 + SiLU*gate, 4 = w2 + residual, 5 = final norm + output head,
- * 6 = the fused layer kernel (2, 3, 4 and the next layer's 0 as one launch).
+ * 2 = wo + residual, 3 = ffn_norm + w1|w3 + SiLU*gate, 4 = w2 + residual, 5 = final norm + output head.
  * bytes_per_launch (may be NULL): the algorithmic bytes of one launch (weights once + vectors).
  * The launches use the model's token-step state and activation buffers as they are and leave them overwritten (position
  * T - 1, a fixed token id), and which = 0 writes the K / V rows of position T - 1 of every layer of `caches`: use caches

@@ -87,6 +87,7 @@ def lib() -> C.CDLL:
         "orc_get_threads": (C.c_int, []),
         "orc_set_reference_threading": (None, [C.c_int]),
         "orc_set_alt_order": (None, [C.c_int]),
+        "orc_set_exact_sums": (None, [C.c_int]),
         "orc_model_create": (vp, [C.POINTER(Params)]),
         "orc_model_free": (None, [vp]),
         "orc_model_set_tensor": (C.c_int, [vp, C.c_int, C.c_int, vp, C.c_int, C.c_int, C.c_int]),
@@ -269,6 +270,11 @@ def set_threads(n: int) -> None:
 def set_alt_order(on: bool) -> None:
     """Sensitivity probe: f16 projections summed in another valid fp32 order (NOT the reference's values)."""
     lib().orc_set_alt_order(1 if on else 0)
+
+
+def set_exact_sums(on: bool) -> None:
+    """Second probe: every sum accumulated in float64 and rounded once (NOT the reference's values; same rounding points)."""
+    lib().orc_set_exact_sums(1 if on else 0)
 
 
 def set_reference_threading(on: bool) -> None:

@@ -154,6 +154,49 @@ static inline float hsum8_alt(__m256 ymm) {
     return t;
 }
 
+/* Second probe, off by default (orc_set_exact_sums): every sum of products or of terms -- the dot products of the
+ * projections, of the scores, of P.V and of the output head, the sum of squares of RMSNorm, the softmax denominator -- is
+ * accumulated in float64 (products of f16 or f32 operands are exact in float64; the additions then carry a relative error
+ * of 1e-16, nothing beside fp32's 6e-8) and rounded to f32 once.  Everything else is as in the reference's arithmetic: the
+ * same f16 rounding points, the same f32 element-wise steps, the same libm calls.  The values are NOT the reference's:
+ * they are what its arithmetic would give if no fp32 addition inside a sum rounded, i.e. the point that the reference and
+ * any reordering of its additions scatter around.  Pinned by tests/test_oracle.py against math.fsum. */
+static int g_exact = 0;
+void orc_set_exact_sums(int on) { g_exact = on ? 1 : 0; }
+
+static inline double hsum4d(__m256d v) {
+    double l[4];
+    _mm256_storeu_pd(l, v);
+    return (l[0] + l[1]) + (l[2] + l[3]);
+}
+
+static double dotd_f32(const float *a, const float *b, int k) {
+    __m256d s0 = _mm256_setzero_pd(), s1 = s0;
+    int p = 0;
+    for (; p + 8 <= k; p += 8) {
+        __m256 av = _mm256_loadu_ps(a + p), bv = _mm256_loadu_ps(b + p);
+        s0 = _mm256_fmadd_pd(_mm256_cvtps_pd(_mm256_castps256_ps128(av)), _mm256_cvtps_pd(_mm256_castps256_ps128(bv)), s0);
+        s1 = _mm256_fmadd_pd(_mm256_cvtps_pd(_mm256_extractf128_ps(av, 1)), _mm256_cvtps_pd(_mm256_extractf128_ps(bv, 1)), s1);
+    }
+    double t = hsum4d(_mm256_add_pd(s0, s1));
+    for (; p < k; p++) t += (double)a[p] * (double)b[p];
+    return t;
+}
+
+static double dotd_f16(const uint16_t *a, const uint16_t *b, int k) {
+    __m256d s0 = _mm256_setzero_pd(), s1 = s0;
+    int p = 0;
+    for (; p + 8 <= k; p += 8) {
+        __m256 av = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(a + p)));
+        __m256 bv = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(b + p)));
+        s0 = _mm256_fmadd_pd(_mm256_cvtps_pd(_mm256_castps256_ps128(av)), _mm256_cvtps_pd(_mm256_castps256_ps128(bv)), s0);
+        s1 = _mm256_fmadd_pd(_mm256_cvtps_pd(_mm256_extractf128_ps(av, 1)), _mm256_cvtps_pd(_mm256_extractf128_ps(bv, 1)), s1);
+    }
+    double t = hsum4d(_mm256_add_pd(s0, s1));
+    for (; p < k; p++) t += (double)_cvtsh_ss(a[p]) * (double)_cvtsh_ss(b[p]);
+    return t;
+}
+
 static inline float hsum8_v(__m256 ymm) {
     /* simd_support.rs:97-105, instruction for instruction */
     __m256 ymm2 = _mm256_permute2f128_ps(ymm, ymm, 1);
@@ -166,6 +209,7 @@ static inline float hsum8_v(__m256 ymm) {
 float orc_hsum8(const float a[8]) { return hsum8_v(_mm256_loadu_ps(a)); }
 
 float orc_dot8_f32(const float *a, const float *b, int k) {
+    if (g_exact) return (float)dotd_f32(a, b, k);
     __m256 acc = _mm256_setzero_ps();
     int p = 0;
     for (; p + 8 <= k; p += 8) {
@@ -203,6 +247,7 @@ float orc_dot8_f32_scalar(const float *a, const float *b, int k) {
 static inline __m256 load8_f16(const uint16_t *p) { return _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)p)); }
 
 float orc_dot8_f16(const uint16_t *a, const uint16_t *b, int k) {
+    if (g_exact) return (float)dotd_f16(a, b, k);
     __m256 acc = _mm256_setzero_ps();
     int p = 0;
     for (; p + 8 <= k; p += 8) {
@@ -222,6 +267,13 @@ float orc_dot8_f16(const uint16_t *a, const uint16_t *b, int k) {
 /* Four weight rows against one x row, sharing the x loads: the value per output is dot8. */
 static inline void dot8x4_f16(const uint16_t *x, const uint16_t *w0, const uint16_t *w1, const uint16_t *w2,
                               const uint16_t *w3, int k, float out[4]) {
+    if (g_exact) { /* not the reference's values: see orc_set_exact_sums */
+        out[0] = (float)dotd_f16(x, w0, k);
+        out[1] = (float)dotd_f16(x, w1, k);
+        out[2] = (float)dotd_f16(x, w2, k);
+        out[3] = (float)dotd_f16(x, w3, k);
+        return;
+    }
     __m256 a0 = _mm256_setzero_ps(), a1 = a0, a2 = a0, a3 = a0;
     int p = 0;
     if (g_alt_order) { /* not the reference's order: see orc_set_alt_order */
@@ -281,6 +333,13 @@ static inline void dot8x4_f16(const uint16_t *x, const uint16_t *w0, const uint1
 
 static inline void dot8x4_f32(const float *x, const float *w0, const float *w1, const float *w2, const float *w3,
                               int k, float out[4]) {
+    if (g_exact) {
+        out[0] = (float)dotd_f32(x, w0, k);
+        out[1] = (float)dotd_f32(x, w1, k);
+        out[2] = (float)dotd_f32(x, w2, k);
+        out[3] = (float)dotd_f32(x, w3, k);
+        return;
+    }
     __m256 a0 = _mm256_setzero_ps(), a1 = a0, a2 = a0, a3 = a0;
     int p = 0;
     for (; p + 8 <= k; p += 8) {
@@ -377,6 +436,12 @@ void orc_matmul_f32_seqk(const float *a, int m, const float *b, int n, int k, fl
      * blocking over rows/cols/k only changes the order in which different elements are visited. */
     for (int i = 0; i < m; i++) {
         for (int c = 0; c < n; c++) {
+            if (g_exact) {
+                double accd = 0.0;
+                for (int kk = 0; kk < k; kk++) accd += (double)a[(size_t)i * k + kk] * (double)b[(size_t)kk * n + c];
+                out[(size_t)i * n + c] = (float)accd;
+                continue;
+            }
             float acc = 0.0f;
             for (int kk = 0; kk < k; kk++) {
                 acc = fmaf(a[(size_t)i * k + kk], b[(size_t)kk * n + c], acc);
@@ -389,6 +454,12 @@ void orc_matmul_f32_seqk(const float *a, int m, const float *b, int n, int k, fl
 void orc_vector_matrix_mul_f32(const float *a, const float *b, int k, int n, float *out) {
     /* tensor.rs:1954-1980: lane i of sum8 accumulates rows (row8*8 + i); rows past k contribute zeros. */
     for (int c = 0; c < n; c++) {
+        if (g_exact) {
+            double accd = 0.0;
+            for (int row = 0; row < k; row++) accd += (double)a[row] * (double)b[(size_t)row * n + c];
+            out[c] = (float)accd;
+            continue;
+        }
         float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (int row = 0; row < k; row += 8) {
             for (int i = 0; i < 8; i++) {
@@ -410,9 +481,15 @@ void orc_rmsnorm_row(const float *x, const float *w, int d, double eps, float *o
      * .hadamard_product_broadcast(weight)   (transformer.rs:476-480; tensor.rs:537-547, 511-522, 595-605,
      * 561-571, 619-636, 654-677).  Every intermediate is an f32 tensor. */
     float sum = 0.0f;
-    for (int i = 0; i < d; i++) {
-        float sq = x[i] * x[i];
-        sum += sq;
+    if (g_exact) {
+        double sd = 0.0;
+        for (int i = 0; i < d; i++) sd += (double)x[i] * (double)x[i];
+        sum = (float)sd;
+    } else {
+        for (int i = 0; i < d; i++) {
+            float sq = x[i] * x[i];
+            sum += sq;
+        }
     }
     float mean = sum / (float)d;
     float inner = mean + (float)eps;
@@ -425,7 +502,13 @@ void orc_rmsnorm_row(const float *x, const float *w, int d, double eps, float *o
 
 void orc_softmax_row(const float *s, int n, float *out) {
     float sum = 0.0f;
-    for (int i = 0; i < n; i++) sum += expf(s[i]);
+    if (g_exact) {
+        double sd = 0.0;
+        for (int i = 0; i < n; i++) sd += (double)expf(s[i]);
+        sum = (float)sd;
+    } else {
+        for (int i = 0; i < n; i++) sum += expf(s[i]);
+    }
     for (int i = 0; i < n; i++) out[i] = expf(s[i]) / sum;
 }
 

@@ -120,6 +120,10 @@ void orc_set_reference_threading(int on);
 /* Sensitivity probe (default off): the f16 projections sum their products in another valid fp32 order (not the reference's).
  * Measures how far the reference's own results move under a reordering of its additions. */
 void orc_set_alt_order(int on);
+/* Second probe (default off): every sum (dot products, RMSNorm's sum of squares, the softmax denominator) accumulated in float64
+ * and rounded to f32 once; rounding points, element-wise steps and libm calls unchanged.  NOT the reference's values: the point
+ * that the reference and every reordering of its fp32 additions scatter around. */
+void orc_set_exact_sums(int on);
 
 orc_model *orc_model_create(const orc_params *p);
 void       orc_model_free(orc_model *m);

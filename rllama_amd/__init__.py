@@ -50,6 +50,10 @@ class Context:
 
     sync = flush
 
+    def set_option(self, name: str, value=None) -> None:
+        """One of the library's switches (NAME of the RLLAMA_HIP_<NAME> variables rlh_init reads once); None = its default."""
+        check(self._lib.rlh_set_option(self._h, name.encode(), None if value is None else str(value).encode()))
+
     def device_info(self):
         name = C.create_string_buffer(256)
         cus = C.c_int()
@@ -256,7 +260,6 @@ class Transformer:
         return out, ms.value
 
     STEP_KERNELS = ("qkv_rope_kvwrite", "attn_decode", "wo_residual", "w13_silu", "w2_residual", "head")
-    FUSED_LAYER_KERNEL = 6   # wo + w1|w3 + w2 + the next layer's wq|wk|wv as one launch
 
     def time_kernel(self, which: int, T: int, iters: int, caches: TransformerCaches):
         """(microseconds per launch, algorithmic bytes per launch) of one token-step kernel, HIP-event timed."""

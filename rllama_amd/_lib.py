@@ -46,6 +46,7 @@ SIGNATURES = {
     "rlh_shutdown": (None, [_vp]),
     "rlh_sync": (C.c_int, [_vp]),
     "rlh_last_error": (C.c_char_p, []),
+    "rlh_set_option": (C.c_int, [_vp, C.c_char_p, C.c_char_p]),
     "rlh_device_info": (C.c_int, [_vp, C.c_char_p, C.c_int, _ip, C.POINTER(C.c_uint64)]),
     "rlh_model_create": (C.c_int, [_vp, C.POINTER(ModelParams), _vpp]),
     "rlh_model_free": (None, [_vp]),

@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "_obj")
 LIB = os.path.join(HERE, "librllama_hip.so")
 
-SOURCES = ["gemv.hip", "decode_fused.hip", "attention.hip", "gemm.hip", "gemm_dma.hip", "gemm_kgroup.hip", "attn_prefill.hip", "prefill.hip", "prefill_f32.hip", "misc.hip", "sampler.hip", "api.hip", "api_ops.hip"]
+SOURCES = ["gemv.hip", "attention.hip", "gemm.hip", "gemm_dma.hip", "gemm_kgroup.hip", "attn_prefill.hip", "prefill.hip", "prefill_f32.hip", "misc.hip", "sampler.hip", "api.hip", "api_ops.hip"]
 HEADERS = ["kernels.h", "device_utils.h", "gemv_device.h", "gemm_epilogue.h", "synth.h", "api_internal.h", os.path.join("..", "..", "include", "rllama_hip.h")]  # relative to csrc/
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"

@@ -71,6 +71,7 @@ struct PrefillScratch {
     void *xn = nullptr, *qkv = nullptr, *q2 = nullptr, *v_t = nullptr, *p2 = nullptr, *a = nullptr;
     void *g = nullptr, *u = nullptr, *mm = nullptr;
     void *gemm_ws = nullptr; // fp32 partial sums of split-K products (short prompts)
+    bool gemm_attention = false; // the buffers of the two-GEMM form of attention (scores, p2) exist
     static constexpr size_t kGemmWsBytes = (size_t)64 << 20;
     void release() {
         void *all[] = {x, h, scores, xn, qkv, q2, v_t, p2, a, g, u, mm, gemm_ws};
@@ -103,27 +104,13 @@ struct rlh_model {
     float *attn_ws = nullptr;
     unsigned *attn_tickets = nullptr; // [n_heads] arrival counters of the in-kernel merge (zero between launches)
     int max_splits = kAttnDecodeMaxSplits;
-    int attn_single_max = 384; // sequence lengths up to this use one block per head
-    int attn_chunk = 128;      // positions per block beyond that
-    int attn_merge_mode = 2;   // how the blocks of a split sequence are merged (AttnDecodeParams::merge_mode)
     bool capturing = false;    // a decode step is being recorded into a HIP graph
-    // fused layer kernel (decode_fused.hip), RLLAMA_HIP_FUSED=1; otherwise one launch per matrix-vector product
-    bool fused_layers = getenv("RLLAMA_HIP_FUSED") && atoi(getenv("RLLAMA_HIP_FUSED")) != 0;
-    FusedBarrierState *fused_barrier = nullptr; // one per kernel variant: a barrier's counters assume one grid size for its lifetime
-    // bound of every barrier wait: 200 ms at the 100 MHz wall clock (RLLAMA_HIP_FUSED_LIMIT_TICKS overrides it; tests use 0)
-    long long fused_limit_ticks = getenv("RLLAMA_HIP_FUSED_LIMIT_TICKS") ? atoll(getenv("RLLAMA_HIP_FUSED_LIMIT_TICKS")) : 20000000;
-    int fused_blocks[4] = {0, 0, 0, 0};     // grid per kernel variant (last phase wq|wk|wv / f16 head / f32 head / none), 0 = not yet asked
-    bool fused_used = false;                // a fused kernel was enqueued since the error word was last checked
-    bool attn_lds_stage = getenv("RLLAMA_HIP_ATTN_LDS") && atoi(getenv("RLLAMA_HIP_ATTN_LDS")) != 0; // comparison variant of the decode attention
     int stream_weights = 1;
     PrefillScratch pf;
     int prefill_mode = 0; // 0: matrix-core prefill where available (f16 mode), 1: token by token
-    // fused attention kernel for multi-token calls (head_dim 64 / 128); RLLAMA_HIP_PREFILL_ATTN=gemm keeps the two-GEMM path
-    bool prefill_attn_fused = !(getenv("RLLAMA_HIP_PREFILL_ATTN") && !strcmp(getenv("RLLAMA_HIP_PREFILL_ATTN"), "gemm"));
-    int prefill_attn_parts = getenv("RLLAMA_HIP_PREFILL_ATTN_PARTS") && atoi(getenv("RLLAMA_HIP_PREFILL_ATTN_PARTS")) == 4 ? 4 : 2;
-    // with two workgroups per compute unit (the four-wavefront form, the default) the second half of the grid runs upwards from
-    // the lightest query block; with one (the eight-wavefront form) the heaviest blocks go first
-    int prefill_attn_order = getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER") ? atoi(getenv("RLLAMA_HIP_PREFILL_ATTN_ORDER")) : (prefill_attn_parts == 2 ? 2 : 1);
+    // the greedy pick inside the output head's launch: one record per workgroup, one arrival counter (zero between launches)
+    float *amax_ws = nullptr;
+    unsigned *amax_ticket = nullptr;
     // host mirror of the device state after a greedy call: next position to fill, or -1 if the device holds no sampled token
     uint64_t uid = 0;   // unique per created model: a later model at the same address is still another model
     int next_pos = -1;
@@ -147,7 +134,66 @@ struct rlh_caches {
     int f16 = 0;
     // one captured decode step (token step + greedy pick) per attention grid shape, replayed by the greedy loops
     std::map<int, hipGraphExec_t> step_graphs;
+    unsigned graphs_tun_version = 0; // the context's switches when the graphs were captured
 };
+
+// ------------------------------------------------------------------------------------------------
+// switches
+// ------------------------------------------------------------------------------------------------
+namespace rlh {
+bool tunables_set(Tunables &t, const char *name, const char *value) {
+    if (!name) return false;
+    const Tunables dflt;
+    const std::string n(name);
+    const bool reset = value == nullptr;
+    const int v = reset ? 0 : atoi(value);
+    auto flag_off = [&](int &no_field) { no_field = reset ? 0 : (v == 0 ? 1 : 0); return true; }; // NAME=0 switches a default-on feature off
+    if (n == "GEMV_BURST") return flag_off(t.gemv_burst_fixed);
+    if (n == "ATTN_CHUNK") { t.attn_chunk = reset ? dflt.attn_chunk : v; return reset || v == 0 || v == -1 || v >= 16; }
+    if (n == "ATTN_SINGLE_MAX") { t.attn_single_max = reset ? dflt.attn_single_max : v; return reset || v >= 0; }
+    if (n == "ATTN_MERGE") { t.attn_merge_mode = reset ? dflt.attn_merge_mode : v; return reset || v == 0 || v == 2; }
+    if (n == "ATTN_LDS") { t.attn_lds = reset ? 0 : (v != 0); return true; }
+    if (n == "PREFILL_ATTN") { t.prefill_attn_gemm = !reset && !strcmp(value, "gemm"); return reset || !strcmp(value, "gemm") || !strcmp(value, "fused"); }
+    if (n == "PREFILL_ATTN_ORDER") { t.prefill_attn_order = reset ? dflt.prefill_attn_order : v; return reset || (v >= 0 && v <= 2); }
+    if (n == "DECODE_GRAPH") { t.decode_graph = reset ? 0 : (v != 0); return true; }
+    if (n == "DECODE_FOLD") { t.decode_fold = reset ? 1 : (v != 0); return true; }
+    if (n == "GEMM_TILE") { t.gemm.tile_plus1 = reset ? 0 : v + 1; return reset || (v >= 0 && v <= 3); }
+    if (n == "GEMM_SPLIT_K") { t.gemm.split_k = reset ? 0 : v; return reset || v >= 0; }
+    if (n == "GEMM_SPLIT_HALF") return flag_off(t.gemm.no_split_half);
+    if (n == "GEMM_DUAL") { t.gemm.dual_plus1 = reset ? 0 : v + 1; return reset || (v >= 0 && v <= 5); }
+    if (n == "GEMM_DUAL_CUT") return flag_off(t.gemm.no_dual_cut);
+    if (n == "GEMM_ROPE") return flag_off(t.gemm.no_rope_epilogue);
+    if (n == "FINISH_NORM") return flag_off(t.gemm.no_finish_norm);
+    if (n == "GEMM_KGROUP") return flag_off(t.gemm.no_kgroup);
+    return false;
+}
+
+void tunables_from_env(Tunables &t) {
+    static const char *const names[] = {"GEMV_BURST", "ATTN_CHUNK", "ATTN_SINGLE_MAX", "ATTN_MERGE", "ATTN_LDS", "PREFILL_ATTN", "PREFILL_ATTN_ORDER",
+                                        "DECODE_GRAPH", "DECODE_FOLD", "GEMM_TILE", "GEMM_SPLIT_K", "GEMM_SPLIT_HALF", "GEMM_DUAL", "GEMM_DUAL_CUT",
+                                        "GEMM_ROPE", "FINISH_NORM", "GEMM_KGROUP"};
+    for (const char *name : names) {
+        const std::string env = std::string("RLLAMA_HIP_") + name;
+        const char *val = getenv(env.c_str());
+        if (val != nullptr && !tunables_set(t, name, val)) {
+            (void)tunables_set(t, name, nullptr); // an unusable value leaves the default in place
+            fprintf(stderr, "rllama_hip: ignoring %s=%s\n", env.c_str(), val);
+        }
+    }
+}
+} // namespace rlh
+
+extern "C" int rlh_set_option(rlh_ctx *ctx, const char *name, const char *value) {
+    if (!ctx || !name) return fail(RLH_ERR_INVALID, "rlh_set_option: NULL argument");
+    CtxLock lock(ctx);
+    Tunables t = ctx->tun;
+    if (!tunables_set(t, name, value)) return fail(RLH_ERR_INVALID, "rlh_set_option: unknown option or unusable value: %s=%s", name, value ? value : "(default)");
+    // work queued under the old setting finishes first: captured decode steps and work buffers depend on some of these
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    ctx->tun = t;
+    ctx->tun_version++;
+    return RLH_OK;
+}
 
 // ------------------------------------------------------------------------------------------------
 // context
@@ -166,6 +212,7 @@ extern "C" int rlh_init(int device_ordinal, int verbose, rlh_ctx **out) {
     rlh_ctx *c = new rlh_ctx();
     c->device = device_ordinal;
     c->verbose = verbose;
+    tunables_from_env(c->tun); // the only place the library reads its environment switches
     if ((e = hipSetDevice(device_ordinal)) != hipSuccess || (e = hipGetDeviceProperties(&c->prop, device_ordinal)) != hipSuccess) {
         delete c;
         return fail(RLH_ERR_HIP, "rlh_init: %s", hipGetErrorString(e));
@@ -271,18 +318,6 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     m->prm = *prm;
     m->prm.percentage_to_gpu = clamp_percentage(prm->percentage_to_gpu);
     m->head_dim = hd;
-    if (const char *e = getenv("RLLAMA_HIP_ATTN_CHUNK")) { // tuning knobs: positions per attention block / single-block limit
-        const int v = atoi(e);
-        if (v >= 16) m->attn_chunk = v;
-    }
-    if (const char *e = getenv("RLLAMA_HIP_ATTN_SINGLE_MAX")) {
-        const int v = atoi(e);
-        if (v >= 0) m->attn_single_max = v;
-    }
-    if (const char *e = getenv("RLLAMA_HIP_ATTN_MERGE")) {
-        const int v = atoi(e);
-        if (v >= 0 && v <= 2) m->attn_merge_mode = v;
-    }
     // transformer.rs:266-268
     m->last_layer_on_gpu = (int)std::round(m->prm.percentage_to_gpu * (float)(prm->n_layers - 1));
     m->n_resident = m->last_layer_on_gpu + 1;
@@ -345,7 +380,8 @@ extern "C" int rlh_model_create(rlh_ctx *ctx, const rlh_model_params *prm, rlh_m
     B((void **)&m->prompt_dev, sizeof(int32_t) * m->prompt_cap);
     B((void **)&m->attn_ws, sizeof(float) * attn_decode_workspace_floats(prm->n_heads, hd, m->max_splits));
     B((void **)&m->attn_tickets, sizeof(unsigned) * (size_t)prm->n_heads);
-    B((void **)&m->fused_barrier, sizeof(FusedBarrierState) * 4);
+    B((void **)&m->amax_ws, gemv_argmax_ws_bytes());
+    B((void **)&m->amax_ticket, 256);
     if (rc == RLH_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(RLH_ERR_HIP, "rlh_model_create: hipDeviceSynchronize failed");
     if (rc != RLH_OK) {
         rlh_model_free(m);
@@ -372,7 +408,7 @@ extern "C" void rlh_model_free(rlh_model *m) {
     free_weight(m->norm);
     free_weight(m->output);
     m->pf.release();
-    void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws, m->attn_tickets, m->fused_barrier};
+    void *bufs[] = {m->freqs, m->x, m->h, m->q, m->att, m->att_o, m->mh, m->ffn_o, m->logits, m->state, m->out_tokens, m->prompt_dev, m->attn_ws, m->attn_tickets, m->amax_ws, m->amax_ticket};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -662,19 +698,26 @@ extern "C" int rlh_caches_read(const rlh_caches *c, int layer, int head, int whi
 // ------------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------------
-static int attn_splits(const rlh_model *m, int T) { return attn_splits_rule(T, m->attn_single_max, m->attn_chunk, m->max_splits); }
+static int attn_splits(const rlh_model *m, int T) {
+    const Tunables &t = m->ctx->tun;
+    return attn_splits_rule(T, m->prm.n_heads, m->ctx->prop.multiProcessorCount, t.attn_single_max, t.attn_chunk, m->max_splits);
+}
 
 enum StepKernel { kStepQkv = 0, kStepAttn = 1, kStepWo = 2, kStepW13 = 3, kStepW2 = 4, kStepHead = 5 };
 
 // The launch parameters of one matrix-vector kernel of layer l (or of the output head) for the token described by the
 // device state; *epi receives its epilogue.  which: kStepQkv, kStepWo, kStepW13, kStepW2, kStepHead.
-static void build_gemv_step(rlh_model *m, rlh_caches *c, int l, int which, int first_layer, GemvParams *out, int *epi) {
+// from_embedding: layer 0 of a whole token step reads its input row from the embedding table (no launch of its own for it);
+// pick: the output head also makes the greedy pick and advances the token-step state.
+static void build_gemv_step(rlh_model *m, rlh_caches *c, int l, int which, int first_layer, GemvParams *out, int *epi, bool from_embedding = false,
+                            bool pick = false) {
     const rlh_model_params &P = m->prm;
     const int d = P.dim, F = P.ffn_hidden, V = P.vocab_size;
     const int f16 = P.force_f16 ? 1 : 0;
     const float eps = (float)P.norm_eps; // add_scalar(self.eps as f32), transformer.rs:477
     GemvParams g{};
     g.stream_weights = m->stream_weights;
+    g.burst_fixed = m->ctx->tun.gemv_burst_fixed;
     g.w_is_f16 = f16;
     g.x_f16 = f16;
     g.round_y = f16;
@@ -686,6 +729,7 @@ static void build_gemv_step(rlh_model *m, rlh_caches *c, int l, int which, int f
         // (transformer.rs:445, 378-381; tensor.rs:1837-1918)
         GemvParams p{};
         p.stream_weights = m->stream_weights;
+        p.burst_fixed = m->ctx->tun.gemv_burst_fixed;
         p.w = m->output.p;
         p.w_is_f16 = m->output.f16;
         p.x = m->h;
@@ -697,8 +741,16 @@ static void build_gemv_step(rlh_model *m, rlh_caches *c, int l, int which, int f
         p.y = m->logits;
         p.n_rows = V;
         p.k = d;
-        *out = p;
         *epi = kEpiStore;
+        if (pick) {
+            p.amax_ws = m->amax_ws;
+            p.amax_ticket = m->amax_ticket;
+            p.state_rw = m->state;
+            p.out_tokens = m->out_tokens;
+            p.out_cap = m->out_cap;
+            *epi = kEpiStoreArgmax;
+        }
+        *out = p;
         return;
     }
     Layer &L = m->layers[(size_t)l];
@@ -710,7 +762,11 @@ static void build_gemv_step(rlh_model *m, rlh_caches *c, int l, int which, int f
         const size_t layer_elems = (size_t)P.n_heads * P.max_seq_len * m->head_dim;
         const size_t ces = c->f16 ? 2 : 4;
         p.w = L.wqkv.p;
-        if (l == first_layer) {
+        if (l == first_layer && from_embedding) {
+            p.embed_table = m->tok_emb.p; // Embedding::get_embedding (embedding.rs:50-52) inside this launch
+            p.embed_f16 = m->tok_emb.f16;
+            p.x_out = m->x;               // the stream entering the layer, for this layer's first residual add
+        } else if (l == first_layer) {
             p.x = m->x;
         } else {
             p.x = m->h;
@@ -769,14 +825,14 @@ static void build_gemv_step(rlh_model *m, rlh_caches *c, int l, int which, int f
 
 // Enqueues one of the five kernels of layer l (or the output head) for the token described by the device
 // state.  T_host = position + 1 as known to the host (sizes the attention grid).
-static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, int T_host, int first_layer = 0) {
+static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, int T_host, int first_layer = 0, bool from_embedding = false, bool pick = false) {
     hipStream_t st = m->ctx->stream;
     const rlh_model_params &P = m->prm;
     if (which < kStepQkv || which > kStepHead) return fail(RLH_ERR_INVALID, "unknown step kernel %d", which);
     if (which != kStepAttn) {
         GemvParams p;
         int epi = kEpiStore;
-        build_gemv_step(m, c, l, which, first_layer, &p, &epi);
+        build_gemv_step(m, c, l, which, first_layer, &p, &epi, from_embedding, pick);
         if (which == kStepQkv && !m->capturing) p.pos1_host = T_host; // (a captured step is replayed at later positions: it reads the device state)
         HIP_TRY(launch_gemv(p, epi, st));
         return RLH_OK;
@@ -799,91 +855,46 @@ static int enqueue_step_kernel(rlh_model *m, rlh_caches *c, int l, int which, in
     a.round_out = P.force_f16 ? 1 : 0;
     a.workspace = m->attn_ws;
     a.tickets = m->attn_tickets;
-    a.merge_mode = m->attn_merge_mode;
+    a.merge_mode = m->ctx->tun.attn_merge_mode;
     a.chunk_hint = (((T_host + a.n_splits - 1) / a.n_splits) + 15) & ~15;
-    a.lds_stage = m->attn_lds_stage && !m->capturing && c->f16 && (m->head_dim == 128 || m->head_dim == 64) && a.merge_mode == 2 &&
+    a.lds_stage = m->ctx->tun.attn_lds && !m->capturing && c->f16 && (m->head_dim == 128 || m->head_dim == 64) && a.merge_mode == 2 &&
                   (size_t)a.chunk_hint * m->head_dim * 4 <= 128 * 1024;
     HIP_TRY(launch_attn_decode(a, st));
     return RLH_OK;
 }
 
-// The matrix-vector kernels of layer l after its attention -- wo, w1|w3, w2 -- and what follows them (the next layer's
-// wq|wk|wv, or the output head after the last layer when with_head is set) as one launch (decode_fused.hip).
-static int enqueue_fused_layer(rlh_model *m, rlh_caches *c, int l, bool with_head) {
-    FusedLayerParams F{};
-    int epi = 0;
-    build_gemv_step(m, c, l, kStepWo, 0, &F.wo, &epi);
-    build_gemv_step(m, c, l, kStepW13, 0, &F.w13, &epi);
-    build_gemv_step(m, c, l, kStepW2, 0, &F.w2, &epi);
-    const bool last_layer = l + 1 == m->prm.n_layers;
-    F.n_phases = 4;
-    if (!last_layer) {
-        build_gemv_step(m, c, l + 1, kStepQkv, 0, &F.last, &epi);
-        F.last_kind = 0;
-    } else if (with_head) {
-        build_gemv_step(m, c, 0, kStepHead, 0, &F.last, &epi);
-        F.last_kind = m->output.f16 ? 1 : 2;
-    } else {
-        F.n_phases = 3;
-        F.last_kind = 0;
-    }
-    const int variant = F.n_phases == 3 ? 3 : F.last_kind;
-    F.barrier = m->fused_barrier + variant;
-    F.limit_ticks = m->fused_limit_ticks;
-    int &blocks = m->fused_blocks[variant];
-    if (blocks == 0) HIP_TRY(fused_layer_grid(F, m->ctx->prop.multiProcessorCount, &blocks));
-    HIP_TRY(launch_fused_layer(F, blocks, m->ctx->stream));
-    m->fused_used = true;
-    return RLH_OK;
-}
-
-// After the work of a call has completed: did a device-wide barrier of the fused kernel give up?  Then the results of the
-// call are void; the barrier words are cleared so that later calls start clean.
-static int check_fused_barrier(rlh_model *m) {
-    if (!m->fused_used) return RLH_OK;
-    m->fused_used = false;
-    FusedBarrierState host[4];
-    HIP_TRY(hipMemcpy(host, m->fused_barrier, sizeof(host), hipMemcpyDeviceToHost));
-    unsigned err = 0;
-    for (const FusedBarrierState &b : host) err |= b.words[(kFusedGroups + 2) * 32];
-    if (err == 0) return RLH_OK;
-    HIP_TRY(hipMemset(m->fused_barrier, 0, sizeof(host)));
-    m->next_pos = -1;
-    m->greedy_caches = nullptr;
-    return fail(RLH_ERR_HIP, "a device-wide barrier of the fused layer kernel did not complete within its time limit (not every workgroup "
-                             "was resident: is another process using the device?); the call's results are void");
-}
-
 // Enqueues one token step (the body of Transformer::forward for a single row, transformer.rs:361-381):
 // reads state->token / state->pos on the device.
-static int enqueue_token_step(rlh_model *m, rlh_caches *c, int T_host, bool with_head) {
-    HIP_TRY(launch_embed(m->tok_emb.p, m->tok_emb.f16, m->prm.dim, m->state, m->x, m->ctx->stream));
-    if (m->fused_layers) {
-        // wq|wk|wv of layer 0 alone, then per layer: attention, and one launch for everything up to the next attention
-        int rc = enqueue_step_kernel(m, c, 0, kStepQkv, T_host);
-        for (int l = 0; rc == RLH_OK && l < m->prm.n_layers; l++) {
-            rc = enqueue_step_kernel(m, c, l, kStepAttn, T_host);
-            if (rc == RLH_OK) rc = enqueue_fused_layer(m, c, l, with_head);
-        }
-        return rc;
-    }
+static int enqueue_token_step(rlh_model *m, rlh_caches *c, int T_host, bool with_head, bool pick = false) {
+    // pick (with_head only): the greedy pick and the advance of the token-step state follow the head.  With the context's
+    // DECODE_FOLD switch on (default) neither the embedding row nor the pick is a launch of its own.
+    const bool fold = m->ctx->tun.decode_fold != 0;
+    if (!fold) HIP_TRY(launch_embed(m->tok_emb.p, m->tok_emb.f16, m->prm.dim, m->state, m->x, m->ctx->stream));
     for (int l = 0; l < m->prm.n_layers; l++) {
         for (int which = kStepQkv; which <= kStepW2; which++) {
-            int rc = enqueue_step_kernel(m, c, l, which, T_host);
+            int rc = enqueue_step_kernel(m, c, l, which, T_host, 0, fold && l == 0 && which == kStepQkv);
             if (rc != RLH_OK) return rc;
         }
     }
-    if (with_head) return enqueue_step_kernel(m, c, 0, kStepHead, T_host);
+    if (!with_head) return RLH_OK;
+    int rc = enqueue_step_kernel(m, c, 0, kStepHead, T_host, 0, false, pick && fold);
+    if (rc != RLH_OK) return rc;
+    if (pick && !fold) HIP_TRY(launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, m->ctx->stream));
     return RLH_OK;
 }
 
 static int ensure_prefill_scratch(rlh_model *m, int n) {
     PrefillScratch &S = m->pf;
-    if (n <= S.n_cap) return RLH_OK;
-    S.release();
     const size_t d = (size_t)m->prm.dim, F = (size_t)m->prm.ffn_hidden, H = (size_t)m->prm.n_heads, hd = (size_t)m->head_dim;
-    const size_t N = (size_t)n, tp = (N + 127) & ~(size_t)127;
     const size_t es = m->prm.force_f16 ? 2 : 4; // element size of the activations between the GEMMs
+    // the [n x n] score / probability matrices exist only in the GEMM form of attention (the one-kernel form keeps them
+    // on chip); f32 mode turns the scores into probabilities in place
+    const bool gemm_attention = !(es == 2 && !m->ctx->tun.prefill_attn_gemm && attn_prefill_supported((int)hd));
+    if (n <= S.n_cap && (S.gemm_attention || !gemm_attention)) return RLH_OK;
+    if (n < S.n_cap) n = S.n_cap; // (the form of attention changed: same capacity, with the score buffers)
+    HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+    S.release();
+    const size_t N = (size_t)n, tp = (N + 127) & ~(size_t)127;
     hipError_t e = hipSuccess;
     auto A = [&](void **p, size_t bytes) {
         if (e != hipSuccess) return;
@@ -896,9 +907,6 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
     A((void **)&S.qkv, N * 3 * d * es);
     A((void **)&S.q2, N * d * 2 * 2); // f16 mode: hi and lo halves; f32 mode: one float
     A((void **)&S.v_t, H * hd * tp * es);
-    // the [n x n] score / probability matrices exist only in the GEMM form of attention (the one-kernel form keeps them
-    // on chip); f32 mode turns the scores into probabilities in place
-    const bool gemm_attention = !(es == 2 && m->prefill_attn_fused && attn_prefill_supported((int)hd));
     if (gemm_attention) A((void **)&S.scores, H * N * tp * 4);
     if (gemm_attention && es == 2) A((void **)&S.p2, H * N * tp * 2 * 2);
     A((void **)&S.a, N * d * es);
@@ -912,6 +920,7 @@ static int ensure_prefill_scratch(rlh_model *m, int n) {
         return fail(e == hipErrorOutOfMemory ? RLH_ERR_OOM : RLH_ERR_HIP, "prefill work buffers for %d tokens: %s", n, hipGetErrorString(e));
     }
     S.n_cap = n;
+    S.gemm_attention = gemm_attention;
     S.t_pad = (int)tp;
     return RLH_OK;
 }
@@ -941,6 +950,7 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     auto gemm = [&](const void *a, int lda, const void *b, int ldb, void *cc, int ldc, int mm, int nn, int kk, int epi, const float *res,
                     const void *gate = nullptr, const float *norm_w = nullptr, int *norm_done = nullptr) -> int {
         GemmParams g{};
+        g.tune = m->ctx->tun.gemm;
         g.a = (const _Float16 *)a;
         g.b = (const _Float16 *)b;
         g.c = cc;
@@ -983,12 +993,14 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
         rp.head_dim = hd;
         rp.max_seq_len = P.max_seq_len;
         rp.t_pad = tp;
-        const bool fused = m->prefill_attn_fused && attn_prefill_supported(hd);
+        const bool fused = !m->ctx->tun.prefill_attn_gemm && attn_prefill_supported(hd);
         rp.vt_swap = fused ? 1 : 0;
         {
             // wq|wk|wv; RoPE, the hi + lo halves of q, the cache rows and V^T come straight out of the product's epilogue where
             // the shape allows, else the product is stored and a kernel of its own does the same
             GemmParams g{};
+            g.tune = m->ctx->tun.gemm;
+        g.tune = m->ctx->tun.gemm;
             g.a = (const _Float16 *)S.xn;
             g.b = (const _Float16 *)L.wqkv.p;
             g.c = S.qkv;
@@ -1022,8 +1034,7 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
             ap.max_seq_len = P.max_seq_len;
             ap.t_pad = tp;
             ap.scale = 1.0f / sqrtf((float)hd);
-            ap.order = m->prefill_attn_order;
-            ap.key_parts = m->prefill_attn_parts;
+            ap.order = m->ctx->tun.prefill_attn_order;
             HIP_TRY(launch_attn_prefill(ap, st));
         } else {
             // scores[h] = q[h] . K[h]^T summed over the hi and lo parts of q: one pass that skips the tiles above the
@@ -1031,6 +1042,9 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
             const bool one_pass = hd % 64 == 0;
             for (int part = 0; part < (one_pass ? 1 : 2); part++) {
                 GemmParams g{};
+                g.tune = m->ctx->tun.gemm;
+            g.tune = m->ctx->tun.gemm;
+        g.tune = m->ctx->tun.gemm;
                 g.a = (const _Float16 *)S.q2 + (size_t)part * hd;
                 g.b = (const _Float16 *)ck;
                 g.c = S.scores;
@@ -1053,6 +1067,9 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
             {   // out[h] = P[h] . V[h] summed over the hi and lo parts of P, rounded to f16 and written as columns
                 // h * hd .. of the [n x dim] input of wo (the concat of heads and the rounding point of transformer.rs:783-796)
                 GemmParams g{};
+                g.tune = m->ctx->tun.gemm;
+            g.tune = m->ctx->tun.gemm;
+        g.tune = m->ctx->tun.gemm;
                 g.a = (const _Float16 *)S.p2;
                 g.b = (const _Float16 *)S.v_t;
                 g.c = S.a;
@@ -1078,6 +1095,8 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
             // SiLU(w1 x) * (w3 x) with the f16 rounding points of transformer.rs:557-565: where the shape allows, both products
             // in one pass over xn; otherwise w1's product goes to memory and w3's epilogue consumes it
             GemmParams g{};
+            g.tune = m->ctx->tun.gemm;
+        g.tune = m->ctx->tun.gemm;
             g.a = (const _Float16 *)S.xn;
             g.b = (const _Float16 *)L.w1.p;
             g.b2 = (const _Float16 *)L.w3.p;
@@ -1088,6 +1107,8 @@ static int enqueue_prefill(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
             g.lda = g.ldb = d;
             g.ldc = F;
             g.batch = 1;
+            g.workspace = S.gemm_ws; // the same policy as rlh_ffn_gate: whether the pass runs is decided with the work memory in place
+            g.workspace_bytes = PrefillScratch::kGemmWsBytes;
             if (gemm_f16_dual_gate_supported(g)) {
                 HIP_TRY(launch_gemm_f16(g, kGemmEpiSiluGateF16, st));
             } else {
@@ -1146,6 +1167,7 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
     const size_t layer_elems = (size_t)H * P.max_seq_len * hd;
     auto gemm = [&](const void *a, int lda, const void *b, int ldb, float *cc, int ldc, int mm, int nn, int kk, int accumulate) -> int {
         GemmParams g{};
+        g.tune = m->ctx->tun.gemm;
         g.a = (const _Float16 *)a;
         g.b = (const _Float16 *)b;
         g.c = cc;
@@ -1186,6 +1208,8 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
         HIP_TRY(launch_rope_kv_prefill_f32(rp, st));
         {   // scores[h] = q[h] . K[h]^T, tiles above the diagonal skipped (transformer.rs:762-770)
             GemmParams g{};
+            g.tune = m->ctx->tun.gemm;
+        g.tune = m->ctx->tun.gemm;
             g.a = (const _Float16 *)q;
             g.b = (const _Float16 *)ck;
             g.c = S.scores;
@@ -1206,6 +1230,8 @@ static int enqueue_prefill_f32(rlh_model *m, rlh_caches *c, const int32_t *token
         HIP_TRY(launch_causal_softmax_f32(S.scores, H, n, tp, hd, st));
         {   // out[h] = P[h] . V[h], written as columns h * hd .. of the [n x dim] input of wo (transformer.rs:777-796)
             GemmParams g{};
+            g.tune = m->ctx->tun.gemm;
+        g.tune = m->ctx->tun.gemm;
             g.a = (const _Float16 *)S.scores;
             g.b = (const _Float16 *)v_t;
             g.c = att;
@@ -1300,7 +1326,7 @@ extern "C" int rlh_forward(rlh_model *m, rlh_caches *c, const int32_t *tokens, i
     if (rc != RLH_OK) return rc;
     HIP_TRY(hipMemcpyAsync(logits_out, m->logits, sizeof(float) * (size_t)m->prm.vocab_size, hipMemcpyDeviceToHost, m->ctx->stream));
     HIP_TRY(hipStreamSynchronize(m->ctx->stream));
-    return check_fused_barrier(m);
+    return RLH_OK;
 }
 
 // forward + the device pick at top_k = 1 on logits * scale
@@ -1317,7 +1343,7 @@ static int forward_greedy_scaled(rlh_model *m, rlh_caches *c, const int32_t *tok
     HIP_TRY(hipStreamSynchronize(st));
     m->next_pos = start_pos + n;
     m->greedy_caches = c;
-    return check_fused_barrier(m);
+    return RLH_OK;
 }
 
 extern "C" int rlh_forward_greedy(rlh_model *m, rlh_caches *c, const int32_t *tokens, int n, int start_pos, int32_t *next_token) {
@@ -1400,14 +1426,13 @@ extern "C" int rlh_forward_sample(rlh_model *m, rlh_caches *c, const int32_t *to
 // RLLAMA_HIP_DECODE_GRAPH=1 the step is captured once per attention grid shape (the only launch parameter that depends on
 // the host's view of the position) and replayed as a graph.
 static int enqueue_decode_step(rlh_model *m, rlh_caches *c, int T_host) {
-    const char *env = getenv("RLLAMA_HIP_DECODE_GRAPH"); // read per call: a process may switch it between calls
-    const bool use_graph = env != nullptr && atoi(env) != 0;
+    const bool use_graph = m->ctx->tun.decode_graph != 0;
     hipStream_t st = m->ctx->stream;
-    if (!use_graph) {
-        int rc = enqueue_token_step(m, c, T_host, true);
-        if (rc != RLH_OK) return rc;
-        HIP_TRY(launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st));
-        return RLH_OK;
+    if (!use_graph) return enqueue_token_step(m, c, T_host, true, true);
+    if (c->graphs_tun_version != m->ctx->tun_version) { // captured under other switches
+        for (auto &kv : c->step_graphs) (void)hipGraphExecDestroy(kv.second);
+        c->step_graphs.clear();
+        c->graphs_tun_version = m->ctx->tun_version;
     }
     const int key = attn_splits(m, T_host);
     auto it = c->step_graphs.find(key);
@@ -1415,14 +1440,12 @@ static int enqueue_decode_step(rlh_model *m, rlh_caches *c, int T_host) {
         hipGraph_t graph = nullptr;
         HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
         m->capturing = true;
-        int rc = enqueue_token_step(m, c, T_host, true);
+        int rc = enqueue_token_step(m, c, T_host, true, true);
         m->capturing = false;
-        hipError_t e = rc == RLH_OK ? launch_argmax_advance(m->logits, m->prm.vocab_size, m->state, m->out_tokens, m->out_cap, st) : hipSuccess;
         hipError_t e2 = hipStreamEndCapture(st, &graph);
-        if (rc != RLH_OK || e != hipSuccess || e2 != hipSuccess) {
+        if (rc != RLH_OK || e2 != hipSuccess) {
             if (graph) (void)hipGraphDestroy(graph);
             if (rc != RLH_OK) return rc;
-            HIP_TRY(e);
             HIP_TRY(e2);
         }
         hipGraphExec_t exec = nullptr;
@@ -1478,7 +1501,7 @@ extern "C" int rlh_generate_greedy(rlh_model *m, rlh_caches *c, const int32_t *p
     HIP_TRY(e);
     m->next_pos = n_prompt + n_new - 1;
     m->greedy_caches = c;
-    return check_fused_barrier(m);
+    return RLH_OK;
 }
 
 extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32_t *out_tokens, float *ms_total) {
@@ -1516,7 +1539,7 @@ extern "C" int rlh_decode_greedy(rlh_model *m, rlh_caches *c, int n_steps, int32
     HIP_TRY(e2);
     if (ms_total) *ms_total = ms;
     m->next_pos += n_steps;
-    return check_fused_barrier(m);
+    return RLH_OK;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1526,9 +1549,7 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
     if (!m || !c || !us_per_launch || iters < 1) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad argument");
     if (c->model != m || c->model_uid != m->uid) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: caches belong to another model");
     if (!model_ready(m)) return fail(RLH_ERR_STATE, "rlh_model_time_kernel: model has tensors that were never set");
-    constexpr int kStepFused = 6; // wo + w1|w3 + w2 + the next layer's wq|wk|wv as one launch
-    if (T < 1 || T > m->prm.max_seq_len || which < kStepQkv || which > kStepFused) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad T or kernel id");
-    if (which == kStepFused && m->prm.n_layers < 2) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: the fused layer kernel needs two layers");
+    if (T < 1 || T > m->prm.max_seq_len || which < kStepQkv || which > kStepHead) return fail(RLH_ERR_INVALID, "rlh_model_time_kernel: bad T or kernel id");
     CtxLock lock(m->ctx);
     hipStream_t st = m->ctx->stream;
     const uint64_t d = (uint64_t)m->prm.dim, F = (uint64_t)m->prm.ffn_hidden, V = (uint64_t)m->prm.vocab_size;
@@ -1541,7 +1562,6 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
         case kStepWo: *bytes_per_launch = d * d * es + d * 4 + 2 * d * 4; break;
         case kStepW13: *bytes_per_launch = 2 * F * d * es + d * 4 + d * 4 + F * 4; break;
         case kStepW2: *bytes_per_launch = d * F * es + F * 4 + 2 * d * 4; break;
-        case kStepFused: *bytes_per_launch = (4 * d * d + 3 * d * F) * es + 8 * d * 4 + 2 * F * 4 + 2 * d * es; break;
         default: *bytes_per_launch = V * d * (m->output.f16 ? 2 : 4) + d * 4 + d * 4 + V * 4; break;
         }
     }
@@ -1554,8 +1574,7 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
     HIP_TRY(hipEventCreate(&e1));
     int rc = RLH_OK;
     const int L = m->prm.n_layers;
-    // (the fused kernel cycles over layers 0 .. L - 2, whose last phase is the next layer's wq|wk|wv)
-    auto one = [&](int i) { return which == kStepFused ? enqueue_fused_layer(m, c, i % (L - 1), true) : enqueue_step_kernel(m, c, i % L, which, T); };
+    auto one = [&](int i) { return enqueue_step_kernel(m, c, i % L, which, T); };
     for (int i = 0; rc == RLH_OK && i < (L < 4 ? L : 4); i++) rc = one(i); // warm-up
     hipError_t e = hipEventRecord(e0, st);
     for (int i = 0; rc == RLH_OK && e == hipSuccess && i < iters; i++) rc = one(i);
@@ -1568,7 +1587,7 @@ extern "C" int rlh_model_time_kernel(rlh_model *m, rlh_caches *c, int which, int
     if (rc != RLH_OK) return rc;
     HIP_TRY(e);
     *us_per_launch = ms * 1000.0f / (float)iters;
-    return check_fused_barrier(m);
+    return RLH_OK;
 }
 
 extern "C" int rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int round_x, int round_y, int n_buffers, int iters, float *us_per_launch) {
@@ -1600,6 +1619,7 @@ extern "C" int rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int rou
     p.n_rows = rows;
     p.k = k;
     p.stream_weights = 1;
+    p.burst_fixed = ctx->tun.gemv_burst_fixed;
     for (int i = 0; e == hipSuccess && i < n_buffers; i++) {
         p.w = bufs[(size_t)i];
         e = launch_gemv(p, kEpiStore, st);

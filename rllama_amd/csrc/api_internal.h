@@ -37,6 +37,27 @@ struct OpScratch {
 constexpr size_t kOpGemmWsBytes = (size_t)64 << 20;
 constexpr int kOpMaxHeads = 1024;
 
+// The library's switches.  Read from the environment (RLLAMA_HIP_<NAME>) once, when the context is made, and changed
+// afterwards only through rlh_set_option under the context lock: no launch path reads the environment.
+struct Tunables {
+    rlh::GemmTune gemm{};
+    int gemv_burst_fixed = 0;      // GEMV_BURST=0: single-row products always issue bursts of 8 loads per lane
+    int attn_chunk = 0;            // ATTN_CHUNK=N (>= 16): positions per workgroup of a split sequence; 0 = one workgroup per compute unit
+    int attn_single_max = 384;     // ATTN_SINGLE_MAX=N: longest sequence one workgroup per head handles alone
+    int attn_merge_mode = 2;       // ATTN_MERGE=0: the pieces of a split sequence are combined by a second launch; 2: inside the kernel
+    int attn_lds = 0;              // ATTN_LDS=1: cache rows staged through LDS (comparison form)
+    int prefill_attn_gemm = 0;     // PREFILL_ATTN=gemm: multi-token attention as two batched GEMMs around a softmax kernel
+    int prefill_attn_order = 2;    // PREFILL_ATTN_ORDER=0/1/2: launch order of the query blocks of the one-kernel attention
+    int decode_graph = 0;          // DECODE_GRAPH=1: greedy decode loops replay one captured HIP graph per token
+    int decode_fold = 1;           // DECODE_FOLD=0: embedding row and greedy pick as launches of their own instead of inside the first and last product of a token step
+};
+
+namespace rlh {
+// applies NAME=value (value nullptr: back to the default); false if the name or the value is not known
+bool tunables_set(Tunables &t, const char *name, const char *value);
+void tunables_from_env(Tunables &t);
+} // namespace rlh
+
 struct rlh_ctx {
     int device = 0;
     int verbose = 0;
@@ -44,6 +65,8 @@ struct rlh_ctx {
     hipDeviceProp_t prop;
     std::recursive_mutex mu;
     OpScratch ops;
+    Tunables tun;
+    unsigned tun_version = 0;        // bumped by rlh_set_option: captured decode steps of an older version are dropped
     void *noalloc_scratch = nullptr; // this device's address of the library's static work memory (api_ops.hip)
 };
 
@@ -71,5 +94,5 @@ void ops_release(rlh_ctx *ctx); // frees the op-level work memory (rlh_shutdown)
 // device current
 int noalloc_setup(rlh_ctx *ctx);
 // how many blocks per head the decode attention uses at sequence length T
-int attn_splits_rule(int T, int single_max, int chunk, int max_splits);
+int attn_splits_rule(int T, int n_heads, int compute_units, int single_max, int chunk, int max_splits);
 } // namespace rlh

@@ -170,6 +170,7 @@ extern "C" int rlh_gemv(rlh_tensor *y, const rlh_tensor *w, const rlh_tensor *x,
     p.n_rows = w->rows;
     p.k = w->cols;
     p.stream_weights = 1;
+    p.burst_fixed = y->ctx->tun.gemv_burst_fixed;
     HIP_TRY(launch_gemv(p, kEpiStore, y->ctx->stream));
     return RLH_OK;
 }
@@ -188,6 +189,7 @@ extern "C" int rlh_matrix_mul_inplace_transposed(rlh_tensor *dst, const rlh_tens
     if (n > 1 && (f16 || k % 32 == 0)) {
         // more than one row: the matrix-core GEMM (fp32 operands need whole K-tiles of 32, else the per-row path below)
         GemmParams g{};
+        g.tune = dst->ctx->tun.gemm;
         g.a = (const _Float16 *)src->p;
         g.b = (const _Float16 *)other->p;
         g.c = dst->p;
@@ -290,6 +292,7 @@ extern "C" int rlh_ffn_gate(rlh_tensor *dst, const rlh_tensor *x, const rlh_tens
     CtxLock lock(dst->ctx);
     hipStream_t st = dst->ctx->stream;
     GemmParams g{};
+    g.tune = dst->ctx->tun.gemm;
     g.a = (const _Float16 *)x->p;
     g.b = (const _Float16 *)w1->p;
     g.c = dst->p;
@@ -362,11 +365,21 @@ extern "C" int rlh_rope_kvwrite(rlh_tensor *q, const rlh_tensor *k, const rlh_te
 }
 
 namespace rlh {
-int attn_splits_rule(int T, int single_max, int chunk, int max_splits) {
-    // One block per (head, split).  Short sequences stay in one block per head; longer ones are cut into chunks of about
-    // `chunk` positions.
+int attn_splits_rule(int T, int n_heads, int compute_units, int single_max, int chunk, int max_splits) {
+    // One workgroup per (head, split).  Short sequences stay in one workgroup per head; longer ones are cut into pieces of
+    // about `chunk` positions (chunk > 0), or of kAutoChunk positions (chunk == 0, the default), or so that the part holds
+    // about one workgroup per compute unit, in pieces of at least 128 positions (chunk == -1).
+    constexpr int kAutoChunk = 128;
     if (T <= single_max) return 1;
-    int S = (T + chunk - 1) / chunk;
+    int S;
+    if (chunk == -1) {
+        const int per_head = compute_units / (n_heads > 0 ? n_heads : 1);
+        S = (T + 127) / 128;
+        if (S > per_head) S = per_head;
+    } else {
+        const int c = chunk > 0 ? chunk : kAutoChunk;
+        S = (T + c - 1) / c;
+    }
     if (S < 1) S = 1;
     if (S > max_splits) S = max_splits;
     return S;
@@ -417,7 +430,10 @@ static int check_attn_decode(const char *who, const rlh_tensor *out, const rlh_t
     }
     if (T < 1 || T > max_seq_len) return fail(RLH_ERR_STATE, "%s: sequence length %d outside 1..max_seq_len %d", who, T, max_seq_len);
     if (n_heads > kOpMaxHeads) return fail(RLH_ERR_UNSUPPORTED, "%s: more than %d heads", who, kOpMaxHeads);
-    if (*n_splits == 0) *n_splits = attn_splits_rule(T, 384, 128, kAttnDecodeMaxSplits);
+    if (*n_splits == 0) {
+        const Tunables &t = out->ctx->tun;
+        *n_splits = attn_splits_rule(T, n_heads, out->ctx->prop.multiProcessorCount, t.attn_single_max, t.attn_chunk, kAttnDecodeMaxSplits);
+    }
     if (*n_splits < 1 || *n_splits > kAttnDecodeMaxSplits) return fail(RLH_ERR_INVALID, "%s: n_splits %d outside 1..%d", who, *n_splits, kAttnDecodeMaxSplits);
     *head_dim = hd;
     return RLH_OK;
@@ -446,11 +462,7 @@ static hipError_t enqueue_attn_decode(rlh_ctx *ctx, rlh_tensor *out, const rlh_t
     a.round_out = round_out ? 1 : 0;
     a.workspace = ws;
     a.tickets = tickets;
-    a.merge_mode = 2;
-    if (const char *env = getenv("RLLAMA_HIP_ATTN_MERGE")) {
-        const int v = atoi(env);
-        if (v >= 0 && v <= 2) a.merge_mode = v;
-    }
+    a.merge_mode = ctx->tun.attn_merge_mode;
     a.chunk_hint = (((T + n_splits - 1) / n_splits) + 15) & ~15;
     return launch_attn_decode(a, st);
 }
@@ -524,9 +536,7 @@ extern "C" int rlh_attn_prefill(rlh_tensor *out, const rlh_tensor *qkv, rlh_tens
         ap.max_seq_len = max_seq_len;
         ap.t_pad = tp;
         ap.scale = 1.0f / sqrtf((float)hd);
-        const char *parts = getenv("RLLAMA_HIP_PREFILL_ATTN_PARTS"); // 4: the eight-wavefront form (read at every call)
-        ap.key_parts = parts != nullptr && atoi(parts) == 4 ? 4 : 2;
-        ap.order = ap.key_parts == 2 ? 2 : 1;
+        ap.order = ctx->tun.prefill_attn_order;
         e = launch_attn_prefill(ap, st);
     }
     hipError_t e2 = hipStreamSynchronize(st);

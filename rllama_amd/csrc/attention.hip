@@ -58,9 +58,10 @@ __device__ __forceinline__ void unpack8(const uint4_t *raw, float (&out)[8]) {
 // How the partial triples of a split sequence travel from the blocks that make them to the block that merges them.
 enum AttnMergeMode {
     kMergeSeparate = 0, // a second kernel merges (attn_merge_kernel)
-    kMergeFenced = 1,   // last block of a head merges; release / acquire fences at device scope around the ticket
     kMergeThrough = 2   // last block of a head merges; the partials are stored and loaded at device scope (write-through /
-                        // cache-bypassing accesses), the stores only waited for before the ticket
+                        // cache-bypassing accesses), the stores only waited for before the ticket.  (Release / acquire fences
+                        // at device scope around the ticket instead were measured at 48 - 146 us for the same launch: each
+                        // fence writes back or invalidates a whole L2 under the stream.)
 };
 
 template <int kMode>
@@ -239,13 +240,14 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(AttnDecodeParams 
         if (S == 1) return;
         // ---- the block that draws the last ticket of this head merges the head's partial triples ----
         __shared__ int is_last;
-        // every writer makes its stores visible to the device before the block's ticket is drawn
-        if constexpr (kMode == kMergeFenced) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        else { // the write-through stores have left the wavefront (and been acknowledged) before the ticket is drawn
-            asm volatile("" ::: "memory");
-            wait_vmcnt<0>();
-            asm volatile("" ::: "memory");
-        }
+        // The write-through stores have left the wavefront and been acknowledged (vmcnt) before the block's ticket is drawn, and
+        // the merging block reads them with device-scope loads after it.  That an acknowledged device-scope store is visible to
+        // a later device-scope load from another compute unit is a property of this part (gfx950: such stores write through the
+        // XCD's L2 to memory, such loads miss it), not a guarantee of the HIP memory model for relaxed atomics -- there is no
+        // release / acquire edge between the blocks.  rlh_init refuses every other architecture.
+        asm volatile("" ::: "memory");
+        wait_vmcnt<0>();
+        asm volatile("" ::: "memory");
         __syncthreads();
         if (tid == 0) {
             const unsigned prev = __hip_atomic_fetch_add(p.tickets + head, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -255,7 +257,6 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(AttnDecodeParams 
         }
         __syncthreads();
         if (!is_last) return;
-        if constexpr (kMode == kMergeFenced) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         // Every wavefront forms the splits' weights for itself (lane s holds split s), and the first partial outputs are
         // requested before those weights are needed: one memory latency for the whole merge, no exchange through LDS.
         const float *wh = p.workspace + (size_t)head * S * (kHeadDim + 2);
@@ -373,11 +374,12 @@ template <typename CT, int kMode>
 static hipError_t launch_attn_m(const AttnDecodeParams &p, hipStream_t s) {
     // Block shape by the positions a block covers (an upper bound from the host's view of the sequence length): 512 threads
     // cover 64 * 512 / head_dim positions per step of the loop, and the rows of kBatch steps are in flight together, so up to
-    // 8 steps run as one batch (one exposed memory latency); longer chunks loop with batches of 4.
+    // 12 steps run as one batch (one exposed memory latency); longer chunks loop with batches of 4.
     const int chunk = p.chunk_hint > 0 ? p.chunk_hint : p.max_seq_len;
     const int per_step = 8 * 512 / p.head_dim;
     if (chunk <= 2 * per_step) return launch_attn_t<CT, 512, 2, kMode>(p, s);
     if (chunk > 4 * per_step && chunk <= 8 * per_step) return launch_attn_t<CT, 512, 8, kMode>(p, s);
+    if (sizeof(CT) == 2 && chunk > 8 * per_step && chunk <= 12 * per_step) return launch_attn_t<CT, 512, 12, kMode>(p, s);
     return launch_attn_t<CT, 512, 4, kMode>(p, s);
 }
 
@@ -395,7 +397,6 @@ hipError_t launch_attn_decode(const AttnDecodeParams &p, hipStream_t s) {
     hipError_t e;
     switch (p.merge_mode) {
     case kMergeSeparate: e = p.cache_f16 ? launch_attn_m<half_t, kMergeSeparate>(p, s) : launch_attn_m<float, kMergeSeparate>(p, s); break;
-    case kMergeFenced: e = p.cache_f16 ? launch_attn_m<half_t, kMergeFenced>(p, s) : launch_attn_m<float, kMergeFenced>(p, s); break;
     case kMergeThrough: e = p.cache_f16 ? launch_attn_m<half_t, kMergeThrough>(p, s) : launch_attn_m<float, kMergeThrough>(p, s); break;
     default: return hipErrorInvalidValue;
     }

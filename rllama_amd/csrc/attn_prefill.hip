@@ -311,14 +311,11 @@ __global__ __launch_bounds__(128 * KQ, KQ == 2 ? 2 : 1) void attn_prefill_kernel
 bool attn_prefill_supported(int head_dim) { return head_dim == 64 || head_dim == 128; }
 
 hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s) {
-    // key tiles of 64 (four wavefronts) unless asked for the eight-wavefront form; t_pad covers whole key tiles either way
-    const bool four = p.key_parts != 4;
-    if (p.n < 1 || p.n_heads < 1 || (p.t_pad % (four ? 64 : 128)) != 0 || p.t_pad < p.n || (p.dim % 8) != 0 || p.max_seq_len < 1) return hipErrorInvalidValue;
+    // four wavefronts on key tiles of 64; t_pad covers whole key tiles
+    if (p.n < 1 || p.n_heads < 1 || (p.t_pad % 64) != 0 || p.t_pad < p.n || (p.dim % 8) != 0 || p.max_seq_len < 1) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((p.n + kApQueries - 1) / kApQueries * p.n_heads));
-    if (p.head_dim == 64 && four) hipLaunchKernelGGL((attn_prefill_kernel<64, 2>), grid, dim3(256), 0, s, p);
-    else if (p.head_dim == 64) hipLaunchKernelGGL((attn_prefill_kernel<64, 4>), grid, dim3(512), 0, s, p);
-    else if (p.head_dim == 128 && four) hipLaunchKernelGGL((attn_prefill_kernel<128, 2>), grid, dim3(256), 0, s, p);
-    else if (p.head_dim == 128) hipLaunchKernelGGL((attn_prefill_kernel<128, 4>), grid, dim3(512), 0, s, p);
+    if (p.head_dim == 64) hipLaunchKernelGGL((attn_prefill_kernel<64, 2>), grid, dim3(256), 0, s, p);
+    else if (p.head_dim == 128) hipLaunchKernelGGL((attn_prefill_kernel<128, 2>), grid, dim3(256), 0, s, p);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

@@ -137,10 +137,8 @@ hipError_t launch_gemm_f16(const GemmParams &p, int epilogue, hipStream_t s) {
     if (p.m <= 0 || p.n <= 0 || p.k <= 0 || (p.k % 8) != 0 || (p.lda % 8) != 0 || (p.ldb % 8) != 0 || p.batch < 1) return hipErrorInvalidValue;
     if (epilogue == kGemmEpiRopeQkv) return gemm_f16_rope_supported(p) ? launch_gemm_f16_dma(p, epilogue, s) : hipErrorInvalidValue; // fast path only
     if (p.b2 != nullptr) return gemm_f16_dual_gate_supported(p) ? launch_gemm_f16_dma(p, epilogue, s) : hipErrorInvalidValue; // fast path only
-    // RLLAMA_HIP_GEMM_SIMPLE=1 keeps every product on the kernel of this file (tuning / cross-checks)
-    static const bool simple_only = getenv("RLLAMA_HIP_GEMM_SIMPLE") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_SIMPLE")) != 0;
     if (p.k_seg != 0 || p.causal != 0) return gemm_f16_dma_supported(p) ? launch_gemm_f16_dma(p, epilogue, s) : hipErrorInvalidValue;
-    if (!simple_only && gemm_f16_dma_supported(p)) return launch_gemm_f16_dma(p, epilogue, s);
+    if (gemm_f16_dma_supported(p)) return launch_gemm_f16_dma(p, epilogue, s);
     dim3 grid((p.n + kBN - 1) / kBN, (p.m + kBM - 1) / kBM, p.batch);
     switch (epilogue) {
     case kGemmEpiF16: hipLaunchKernelGGL(gemm_f16_kernel<kGemmEpiF16>, grid, dim3(kGemmThreads), 0, s, p); break;

@@ -578,7 +578,7 @@ static int device_compute_units() {
 // Tile choice: time ~ (rounds of workgroups over the compute units) x (work per workgroup) / (efficiency of the tile);
 // larger tiles are more efficient (less L2 -> LDS traffic per flop) but leave compute units idle on small outputs.
 static int choose_tile(const GemmParams &p, double *model_time = nullptr) {
-    static const int forced = getenv("RLLAMA_HIP_GEMM_TILE") ? atoi(getenv("RLLAMA_HIP_GEMM_TILE")) : -1;
+    const int forced = p.tune.tile_plus1 - 1; // -1: by the model below
     if (forced >= 1 && forced <= 3) return forced;
     const int k_halves = p.k * (p.f32_operands ? 2 : 1);
     if (forced == 0 && k_halves % 64 == 0) return 0;
@@ -729,7 +729,7 @@ static int choose_split_k(const GemmParams &p, int tile) {
     if (p.workspace == nullptr || p.batch != 1 || p.k_seg != 0 || p.causal != 0) return 1;
     const int k_halves = p.k * (p.f32_operands ? 2 : 1);
     if (tile != 0 || (p.n % 4) != 0 || (p.ldc % 4) != 0 || k_halves % 64 != 0) return 1;
-    static const int forced = getenv("RLLAMA_HIP_GEMM_SPLIT_K") ? atoi(getenv("RLLAMA_HIP_GEMM_SPLIT_K")) : 0;
+    const int forced = p.tune.split_k;
     const int n_cu = device_compute_units();
     const long blocks = (long)((p.n + 127) / 128) * ((p.m + 127) / 128);
     const int k_tiles = k_halves / 64;
@@ -740,7 +740,7 @@ static int choose_split_k(const GemmParams &p, int tile) {
     // with half the compute units idle as with all of them busy, so two pieces on twice the workgroups nearly halve the product
     // (wo / w2 of the 7B shape at 320 / 384 / 512 rows: 10.0 / 10.7 / 11.1 -> 9.1 / 9.4 / 10.2 ms to the first token; three
     // pieces measured the same as two; at 640 rows and more the tiles fill the part and a cut costs)
-    static const bool half_ok = !(getenv("RLLAMA_HIP_GEMM_SPLIT_HALF") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_SPLIT_HALF")) == 0);
+    const bool half_ok = !p.tune.no_split_half;
     const long max_blocks = p.m > 128 && half_ok ? n_cu / 2 : n_cu / 4;
     if (blocks > max_blocks && forced <= 1) return 1;
     // a single row tile runs its pieces on the 128 x 64 tile: twice the column tiles, half the pieces, half the partial sums
@@ -773,8 +773,7 @@ static hipError_t launch_split_finish(const GemmParams &p, int splits, hipStream
 // rows: 576 = 2.25 rounds of 256), the bit costs a whole round, and as two small products it costs a fraction of one.
 static int choose_dual(const GemmParams &p, int *cut_cols = nullptr) {
     if (cut_cols != nullptr) *cut_cols = 0;
-    const char *env = getenv("RLLAMA_HIP_GEMM_DUAL"); // 0: never, 1 ... 5: that form wherever the kernel can run (tests), unset: by shape; read at every call
-    const int mode = env != nullptr ? atoi(env) : -1;
+    const int mode = p.tune.dual_plus1 - 1; // 0: never, 1 ... 5: that form wherever the kernel can run (tests), -1: by shape
     if (mode == 0 || p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.k % 64 != 0) return 0;
     if ((p.ldc % 8) != 0 || (p.n % 8) != 0 || (reinterpret_cast<uintptr_t>(p.c) % 16) != 0) return 0;
     if (mode >= 1 && mode <= 5) return mode;
@@ -798,7 +797,7 @@ static int choose_dual(const GemmParams &p, int *cut_cols = nullptr) {
     const double dual128 = (double)((blocks128 + n_cu - 1) / n_cu) * 2.0 * 128 * 192 / 0.87;
     // the 256-row form on the columns that make whole rounds, the rest (at most a quarter of a round of its workgroups) as two
     // launches; 3 us per additional launch in the model's unit (6.2e-7 us x K each)
-    static const bool cut_ok = !(getenv("RLLAMA_HIP_GEMM_DUAL_CUT") != nullptr && atoi(getenv("RLLAMA_HIP_GEMM_DUAL_CUT")) == 0);
+    const bool cut_ok = !p.tune.no_dual_cut;
     const long rows256 = (p.m + 255) / 256, full = blocks256 / n_cu, cols_main = full * n_cu / rows256;
     int n1 = 0;
     // (from two whole rounds on: with one, 7B shape 1280 rows and 13B shape 1024 rows, the cut measured 3 % slower than without)
@@ -831,8 +830,7 @@ bool gemm_f16_dual_gate_supported(const GemmParams &p) {
 // The RoPE epilogue needs whole 16-byte pieces everywhere and an unsplit product (a product cut along K has its epilogue in
 // the kernel that adds the partial sums; the caller then stores the product and runs the separate kernel).
 bool gemm_f16_rope_supported(const GemmParams &p) {
-    const char *env = getenv("RLLAMA_HIP_GEMM_ROPE"); // 0: never (the separate kernel); read at every call
-    if (env != nullptr && atoi(env) == 0) return false;
+    if (p.tune.no_rope_epilogue) return false;
     const PrefillRopeParams &R = p.rope;
     if (p.f32_operands || !gemm_f16_dma_supported(p) || p.batch != 1 || p.k_seg != 0 || p.causal != 0 || p.b2 != nullptr) return false;
     if (R.dim <= 0 || R.head_dim <= 0 || p.n != 3 * R.dim || R.n != p.m || R.dim % R.head_dim != 0 || R.head_dim % 8 != 0 || !R.cache_f16) return false;
@@ -890,7 +888,7 @@ hipError_t launch_gemm_f16_dma(const GemmParams &p_in, int epilogue, hipStream_t
         hipError_t e = launch_gemm_f16_dma(q, kGemmEpiF32, s);
         if (e != hipSuccess) return e;
         if (epilogue == kGemmEpiResAddF32 && p_in.norm_w != nullptr && p_in.norm_out != nullptr && p_in.norm_done != nullptr &&
-            p_in.n <= 256 * 4 * kFinishNormVecs && !(getenv("RLLAMA_HIP_FINISH_NORM") && atoi(getenv("RLLAMA_HIP_FINISH_NORM")) == 0)) {
+            p_in.n <= 256 * 4 * kFinishNormVecs && !p_in.tune.no_finish_norm) {
             hipLaunchKernelGGL(gemm_split_finish_norm_kernel, dim3(p_in.m), dim3(256), 0, s, p_in, (const float *)p_in.workspace, splits);
             *p_in.norm_done = 1;
             return hipGetLastError();

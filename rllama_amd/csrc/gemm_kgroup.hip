@@ -303,8 +303,7 @@ __global__ __launch_bounds__(64 * kWM * kWN * kKG) void gemm_f16_kgroup_kernel(G
 }
 
 bool gemm_f16_kgroup_supported(const GemmParams &p, int epilogue, int tile) {
-    const char *env = getenv("RLLAMA_HIP_GEMM_KGROUP"); // 0: never; read at every call
-    if (env != nullptr && atoi(env) == 0) return false;
+    if (p.tune.no_kgroup) return false;
     // tile: the choice of gemm_dma.hip's model -- 0 / 4: 128 x 128.  (256 x 192 tiles with wavefronts of 128 x 96 on every other
     // K-step -- 192 accumulator registers, A fragments single-buffered -- measured 98.8 against 102.2 us on the plain wq|wk|wv product of the 7B shape
     // and 112.4 against 111 us with RoPE and the cache write in the epilogue: the cycles fall as the LDS bytes do, the clock

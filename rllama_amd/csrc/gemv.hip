@@ -39,16 +39,20 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     // (measured: issuing the first burst behind the prologue's loads is worth 1 % on the w1|w3 product, nothing or a loss on
     // the others, so only that instantiation does it)
     constexpr int kPre = (RLH_GEMV_PRELOAD && kEpi == kEpiSilu) ? kPreSelf : kPreNone;
-    uint4_t wpre[1][kBurst];
-    gemv_body<WT, XT, kEpi, kStream, false, kPre, false, 1, kBurst>(p, smem_raw, red, rope_f, wpre, 0u);
+    gemv_body<WT, XT, kEpi, kStream, kPre, kBurst>(p, smem_raw, red, rope_f);
 }
+
+static int gemv_blocks(int n_units) {
+    const int n_waves = n_units < kGemvTargetWaves ? n_units : kGemvTargetWaves;
+    return (n_waves + kGemvWaves - 1) / kGemvWaves;
+}
+
+size_t gemv_argmax_ws_bytes() { return (size_t)gemv_blocks(kGemvTargetWaves) * 16; }
 
 template <typename WT, typename XT, int kEpi>
 static hipError_t launch_gemv_t(GemvParams p, hipStream_t s) {
     constexpr int rows_per_unit = (kEpi == kEpiRopeKv) ? 2 : 1;
-    const int n_units = p.n_rows / rows_per_unit;
-    int n_waves = n_units < kGemvTargetWaves ? n_units : kGemvTargetWaves;
-    const int blocks = (n_waves + kGemvWaves - 1) / kGemvWaves;
+    const int blocks = gemv_blocks(p.n_rows / rows_per_unit);
     const size_t lds = (size_t)gemv_iters(p.k, WVec<WT>::kVec) * kWave * WVec<WT>::kVec * sizeof(XT);
     auto launch = [&](auto kern) -> hipError_t {
         if (lds > 48 * 1024) {
@@ -63,25 +67,20 @@ static hipError_t launch_gemv_t(GemvParams p, hipStream_t s) {
     // dim 6656, ffn 22016 -- have no divisor here and keep the default with its partial last burst).  Same order of additions
     // per lane whatever the burst length, so the same bits.  Measured: w2 of the 7B shape 18.8 -> 17.3 us, wo of the 13B shape
     // 12.2 -> 11.1 us, w2 of the 13B shape 25.7 -> 25.4 us.
-    if constexpr (std::is_same<WT, half_t>::value) {
-        constexpr int mr = GemvShape<WT, kEpi>::kMats * GemvShape<WT, kEpi>::kRows;
-        const char *env = getenv("RLLAMA_HIP_GEMV_BURST"); // 0: always the default length; read at every call
-        const bool fixed = env != nullptr && atoi(env) == 0;
+    if constexpr (std::is_same<WT, half_t>::value && (kEpi == kEpiStore || kEpi == kEpiStoreArgmax)) {
         const int pieces = gemv_iters(p.k, WVec<WT>::kVec);
         auto pick = [&](auto burst) -> hipError_t {
             constexpr int kB = decltype(burst)::value;
             if (p.stream_weights) return launch(gemv_kernel<WT, XT, kEpi, true, kB>);
             return launch(gemv_kernel<WT, XT, kEpi, false, kB>);
         };
-        if (!fixed && pieces % (kGemvBurst / mr) != 0) {
-            // (one matrix, one row per unit only: the 13B shape's wq|wk|wv and w1|w3, 10 pieces per row as 5 + 5 instead of
-            // 4 + 4 + 2 for each of two rows, measured 30.1 against 29.2 us and 46.6 against 46.4 us)
-            if constexpr (mr == 1) {
-                if (pieces % 9 == 0) return pick(std::integral_constant<int, 9>{});
-                if (pieces % 10 == 0) return pick(std::integral_constant<int, 10>{});
-                if (pieces % 11 == 0) return pick(std::integral_constant<int, 11>{});
-                if (pieces % 7 == 0) return pick(std::integral_constant<int, 7>{});
-            }
+        // (one matrix, one row per unit only: the 13B shape's wq|wk|wv and w1|w3, 10 pieces per row as 5 + 5 instead of
+        // 4 + 4 + 2 for each of two rows, measured 30.1 against 29.2 us and 46.6 against 46.4 us)
+        if (!p.burst_fixed && pieces % kGemvBurst != 0) {
+            if (pieces % 9 == 0) return pick(std::integral_constant<int, 9>{});
+            if (pieces % 10 == 0) return pick(std::integral_constant<int, 10>{});
+            if (pieces % 11 == 0) return pick(std::integral_constant<int, 11>{});
+            if (pieces % 7 == 0) return pick(std::integral_constant<int, 7>{});
         }
     }
     if (p.stream_weights) return launch(gemv_kernel<WT, XT, kEpi, true>);
@@ -99,12 +98,17 @@ static hipError_t launch_gemv_e(const GemvParams &p, hipStream_t s) {
 hipError_t launch_gemv(const GemvParams &p, int epilogue, hipStream_t s) {
     const int vec = p.w_is_f16 ? 8 : 4;
     if (p.k < vec || p.n_rows <= 0 || (p.k % vec) != 0) return hipErrorInvalidValue;
+    if (p.embed_table != nullptr && (epilogue != kEpiRopeKv || p.state == nullptr)) return hipErrorInvalidValue;
     switch (epilogue) {
     case kEpiStore: return launch_gemv_e<kEpiStore>(p, s);
     case kEpiSilu: return launch_gemv_e<kEpiSilu>(p, s);
     case kEpiRopeKv:
         if ((p.dim % 2) != 0 || (p.head_dim % 2) != 0 || p.head_dim > 128 || p.n_rows != 3 * p.dim) return hipErrorInvalidValue;
         return launch_gemv_e<kEpiRopeKv>(p, s);
+    case kEpiStoreArgmax:
+        // the output head: fp32 x, no rounding; the pick needs its work memory and the state it advances
+        if (p.x_f16 || p.round_y || !p.amax_ws || !p.amax_ticket || !p.state_rw) return hipErrorInvalidValue;
+        return p.w_is_f16 ? launch_gemv_t<half_t, float, kEpiStoreArgmax>(p, s) : launch_gemv_t<float, float, kEpiStoreArgmax>(p, s);
     default: return hipErrorInvalidValue;
     }
 }

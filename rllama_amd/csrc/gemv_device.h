@@ -1,5 +1,4 @@
-// gemv_device.h -- device code of the batch-1 decode GEMV (gemv.hip has the design notes), shared by the stand-alone
-// kernel (gemv.hip) and the fused layer kernel (decode_fused.hip).
+// gemv_device.h -- device code of the batch-1 decode GEMV (gemv.hip has the design notes).
 #pragma once
 
 #include "kernels.h"
@@ -101,57 +100,11 @@ __device__ __forceinline__ float wave_sum_lane63(float v) {
     return v;
 }
 
-// ---- activations that cross workgroups inside one launch --------------------------------------------------------------
-// Between kernels the launch boundary makes every store visible.  Inside the fused layer kernel an activation vector is
-// written by some workgroups and read by all of them after a device-wide barrier, and the eight L2 caches of the part are
-// not coherent with each other for ordinary accesses: such vectors are stored (kDev) and loaded (kDevLoad) at device scope
-// -- write-through stores that are in memory once acknowledged, loads that do not take a stale L2 line.  Measured
-// alternatives for the reading side: an acquire fence at device scope followed by ordinary loads costs 9 us per barrier
-// (it invalidates the L2 under the weight stream); four-byte device-scope loads cost 3 us per phase (512 workgroups
-// fetching the same few KB dword by dword from memory); 16-byte ones about 1 us.
-// Device-scope 16-byte loads are written as inline assembly (the compiler offers device scope only for scalar types): a
-// batch is issued with act_issue4, then act_wait8 waits for everything outstanding and ties the destination registers to the
-// wait, so that no use of them can be scheduled in front of it.  The ordinary form is a plain load and no wait.
-template <bool kDev>
-__device__ __forceinline__ void act_issue4(float4_t &dst, const float4_t *p) {
-    if constexpr (kDev) asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(dst) : "v"(p) : "memory");
-    else dst = *p;
-}
-template <bool kDev, int kN>
-__device__ __forceinline__ void act_wait(float4_t (&v)[kN]) {
-    static_assert(kN == 8, "batches of eight");
-    if constexpr (kDev)
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])::"memory");
-}
-template <bool kDev>
-__device__ __forceinline__ float act_load1(const float *p) {
-    if constexpr (kDev) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else return *p;
-}
-template <bool kDev>
-__device__ __forceinline__ void act_store4(float4_t *p, float4_t v) {
-    if constexpr (kDev) {
-        float *q = reinterpret_cast<float *>(p);
-        __hip_atomic_store(q, v[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(q + 1, v[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(q + 2, v[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(q + 3, v[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-        *p = v;
-    }
-}
-template <bool kDev>
-__device__ __forceinline__ void act_store1(float *p, float v) {
-    if constexpr (kDev) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *p = v;
-}
-
 // How the first burst of the first row unit reaches the main loop.
 enum GemvPreload {
     kPreNone = 0,   // loaded in the main loop like every other burst
-    kPreSelf = 1,   // issued by the prologue right behind its own loads (they stay ahead of it in the in-order return queue),
+    kPreSelf = 1    // issued by the prologue right behind its own loads (they stay ahead of it in the in-order return queue),
                     // so that its memory latency runs under the norm / staging work
-    kPreGiven = 2   // issued by the caller before this phase began (the fused kernel issues it before the barrier it waits at)
 };
 
 // kBurst: 16-byte loads per lane and burst.  Rows that divide into whole bursts stream about 1 us faster per product than rows
@@ -166,53 +119,60 @@ struct GemvShape {
     static constexpr int kPiece = kWave * kVec;                  // elements one wave-wide load covers
 };
 
-// The bursts of a wavefront in the order its main loop takes them: row units unit_first, unit_first + W, ..., and within a
-// unit the pieces 0, kU, 2 kU, ...  This issues the loads of the first kD of them into wpre and returns a mask of those it
-// issued (bit d: burst d is in wpre[d]); a burst that does not exist or is not a full one (the ragged end of a row) is left
-// to the main loop.  The loads do not depend on x.
-template <typename WT, int kEpi, bool kStream, int kD, int kBurst = kGemvBurst>
-__device__ __forceinline__ unsigned gemv_issue_bursts(const GemvParams &p, uint4_t (&wpre)[kD][kBurst]) {
+// Issues the loads of a wavefront's first burst (pieces 0 .. kU - 1 of its first row unit) into wpre and returns true, or
+// returns false where that burst does not exist or is not a full one (left to the main loop).  The loads do not depend on x.
+template <typename WT, int kEpi, bool kStream, int kBurst = kGemvBurst>
+__device__ __forceinline__ bool gemv_issue_first_burst(const GemvParams &p, uint4_t (&wpre)[kBurst]) {
     using S = GemvShape<WT, kEpi, kBurst>;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int K = p.k;
-    const int pieces = gemv_iters(K, S::kVec);
     const int pieces_full = K / S::kPiece;
     const int n_units = p.n_rows / S::kRows;
-    const int W = gridDim.x * kGemvWaves;
     const WT *wmat[2] = {reinterpret_cast<const WT *>(p.w), reinterpret_cast<const WT *>(p.w_b)};
-    int unit = blockIdx.x * kGemvWaves + wave, c = 0;
-    unsigned mask = 0;
-    static_for<kD>([&](auto dc) {
-        constexpr int d = decltype(dc)::value;
-        if (unit < n_units && c + S::kU <= pieces_full) {
-            mask |= 1u << d;
+    const int unit = blockIdx.x * kGemvWaves + wave;
+    if (unit >= n_units || S::kU > pieces_full) return false;
 #pragma unroll
-            for (int u = 0; u < S::kU; u++)
+    for (int u = 0; u < S::kU; u++)
 #pragma unroll
-                for (int m = 0; m < S::kMats; m++)
+        for (int m = 0; m < S::kMats; m++)
 #pragma unroll
-                    for (int r = 0; r < S::kRows; r++)
-                        wpre[d][(u * S::kMats + m) * S::kRows + r] =
-                            load16<kStream>(wmat[m] + (size_t)(unit * S::kRows + r) * K + (size_t)(c + u) * S::kPiece + lane * S::kVec);
-        }
-        c += S::kU;
-        if (c >= pieces) {
-            c = 0;
-            unit += W;
-        }
-    });
-    return mask;
+            for (int r = 0; r < S::kRows; r++)
+                wpre[(u * S::kMats + m) * S::kRows + r] =
+                    load16<kStream>(wmat[m] + (size_t)(unit * S::kRows + r) * K + (size_t)u * S::kPiece + lane * S::kVec);
+    return true;
+}
+
+// A running greedy candidate: the largest value seen and the lowest id that holds it, and whether a NaN was seen
+// (TokenSampler::sample at top_k = 1, token_sampler.rs:112-147: token 0's value becomes v - v, the rest are untouched).
+struct GreedyBest {
+    float best;
+    int idx;
+    int nan;
+};
+__device__ __forceinline__ void greedy_consider(GreedyBest &g, float v, int i) {
+    if (i == 0) v = v - v;
+    if (v != v) g.nan = 1;
+    if (v > g.best || (g.idx < 0 && v == g.best)) {
+        g.best = v;
+        g.idx = i;
+    }
+}
+__device__ __forceinline__ void greedy_merge(GreedyBest &g, float ov, int oi, int onan) {
+    g.nan |= onan;
+    if (oi >= 0 && (g.idx < 0 || ov > g.best || (ov == g.best && oi < g.idx))) {
+        g.best = ov;
+        g.idx = oi;
+    }
 }
 
 // One GEMV over the whole grid: prologue (x staged in LDS), main loop, epilogue.  `smem_raw` is the block's dynamic LDS
-// (gemv_lds_bytes); `red` 16 floats and `rope_f` 64 float2 of static LDS.  kDev: x / x_add are read and y / x_out written at
-// device scope (see above).  With kPre == kPreGiven, wpre holds the first kD bursts the caller issued and pre_mask says which.
-template <typename WT, typename XT, int kEpi, bool kStream, bool kDev, int kPre, bool kDevLoad = false, int kD = 1, int kBurst = kGemvBurst>
-__device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f, uint4_t (&wpre)[kD][kBurst],
-                                          unsigned pre_mask) {
+// (gemv_lds_bytes); `red` 16 floats and `rope_f` 64 float2 of static LDS.
+template <typename WT, typename XT, int kEpi, bool kStream, int kPre, int kBurst = kGemvBurst>
+__device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f) {
     using S = GemvShape<WT, kEpi, kBurst>;
     constexpr int kVec = S::kVec, kMats = S::kMats, kRows = S::kRows, kU = S::kU, kPiece = S::kPiece;
+    constexpr bool kArgmax = kEpi == kEpiStoreArgmax;
     XT *xs = reinterpret_cast<XT *>(smem_raw);
 
     const int tid = threadIdx.x;
@@ -227,46 +187,71 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     wmat[0] = reinterpret_cast<const WT *>(p.w);
     if constexpr (kMats == 2) wmat[1] = reinterpret_cast<const WT *>(p.w_b);
     const int unit_first = blockIdx.x * kGemvWaves + wave;
+    uint4_t wpre[kBurst];
+    bool have_pre = false;
     auto preload = [&]() {
-        if constexpr (kPre == kPreSelf) pre_mask = gemv_issue_bursts<WT, kEpi, kStream, kD, kBurst>(p, wpre);
+        if constexpr (kPre == kPreSelf) have_pre = gemv_issue_first_burst<WT, kEpi, kStream, kBurst>(p, wpre);
         __builtin_amdgcn_sched_barrier(0);
     };
-    if constexpr (kPre == kPreNone) pre_mask = 0;
 
     // The position and this position's (cos, sin) row are requested first, so that their latencies run under the prologue's
     // (behind it they were two dependent loads in front of the main loop: 1.5 us per launch on the 7B shape).
     int pos = 0;
     [[maybe_unused]] float2 rope_early = make_float2(0.0f, 0.0f);
+    // Layer 0 of a token step takes its input row from the embedding table (Embedding::get_embedding, embedding.rs:50-52:
+    // one table row, widened to f32), named by the token id in the device state: a launch of its own for 16 KB otherwise.
+    [[maybe_unused]] const half_t *emb_h = nullptr;
+    [[maybe_unused]] const float *emb_f = nullptr;
     if constexpr (kEpi == kEpiRopeKv) {
+        if (p.embed_table != nullptr) {
+            const size_t row = (size_t)p.state->token * (size_t)K;
+            if (p.embed_f16) emb_h = reinterpret_cast<const half_t *>(p.embed_table) + row;
+            else emb_f = reinterpret_cast<const float *>(p.embed_table) + row;
+        }
         pos = p.pos1_host > 0 ? p.pos1_host - 1 : p.state->pos;
         const int half_hd = p.head_dim / 2;
         if (tid < half_hd) rope_early = p.freqs[(size_t)pos * half_hd + tid];
     }
+    // four consecutive elements of the input vector
+    auto load_in4 = [&](int i4) -> float4_t {
+        if constexpr (kEpi == kEpiRopeKv) {
+            if (emb_h != nullptr) {
+                typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
+                const half4_t h = *reinterpret_cast<const half4_t *>(emb_h + (size_t)i4 * 4);
+                return float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+            }
+            if (emb_f != nullptr) return *reinterpret_cast<const float4_t *>(emb_f + (size_t)i4 * 4);
+        }
+        return reinterpret_cast<const float4_t *>(p.x)[i4];
+    };
+    auto load_in1 = [&](int i) -> float {
+        if constexpr (kEpi == kEpiRopeKv) {
+            if (emb_h != nullptr) return (float)emb_h[i];
+            if (emb_f != nullptr) return emb_f[i];
+        }
+        return p.x[i];
+    };
 
     // ---- prologue: x = (x_in [+ x_add]) [RMSNorm] [-> f16], staged in LDS, zero padded to kpad ----
     // All global loads of a batch are issued before any is consumed (one exposed memory latency per batch).
     const bool writes_sum = (p.x_out != nullptr) && blockIdx.x == 0;
     const int n4 = K / 4; // k is a multiple of 4
-    const float4_t *x4 = reinterpret_cast<const float4_t *>(p.x);
     const float4_t *a4 = reinterpret_cast<const float4_t *>(p.x_add);
     float4_t *o4 = reinterpret_cast<float4_t *>(p.x_out);
     for (int i = K + tid; i < kpad; i += kGemvThreads) xs[i] = (XT)0.0f;
     if (p.norm_w != nullptr && n4 <= kGemvPrologueVecs * kGemvThreads) {
         // RMSNorm::forward (transformer.rs:476-480): (x * rsqrt(mean(x^2) + eps)) * w, x kept in registers
         const float4_t *w4 = reinterpret_cast<const float4_t *>(p.norm_w);
-        static_assert(kGemvPrologueVecs == 8, "act_wait takes batches of eight");
         float4_t xv[kGemvPrologueVecs], av[kGemvPrologueVecs], wv[kGemvPrologueVecs];
 #pragma unroll
-        for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(xv[j], x4 + min(tid + j * kGemvThreads, n4 - 1));
+        for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = load_in4(min(tid + j * kGemvThreads, n4 - 1));
         if (a4 != nullptr) {
 #pragma unroll
-            for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(av[j], a4 + min(tid + j * kGemvThreads, n4 - 1));
+            for (int j = 0; j < kGemvPrologueVecs; j++) av[j] = a4[min(tid + j * kGemvThreads, n4 - 1)];
         }
 #pragma unroll
         for (int j = 0; j < kGemvPrologueVecs; j++) wv[j] = w4[min(tid + j * kGemvThreads, n4 - 1)];
-        act_wait<kDevLoad>(xv);
         if (a4 != nullptr) {
-            act_wait<kDevLoad>(av);
 #pragma unroll
             for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + av[j]; // transformer.rs:442 / :445
         }
@@ -277,7 +262,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
         for (int j = 0; j < kGemvPrologueVecs; j++) {
             const int i = tid + j * kGemvThreads;
             if (i < n4) {
-                if (writes_sum) act_store4<kDev>(o4 + i, xv[j]);
+                if (writes_sum) o4[i] = xv[j];
 #pragma unroll
                 for (int e = 0; e < 4; e++) ss = fmaf(xv[j][e], xv[j][e], ss);
             }
@@ -297,30 +282,26 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
         preload();
         float ss = 0.0f;
         for (int i = tid; i < K; i += kGemvThreads) {
-            float v = act_load1<kDevLoad>(p.x + i);
-            if (p.x_add != nullptr) v = v + act_load1<kDevLoad>(p.x_add + i);
-            if (writes_sum) act_store1<kDev>(p.x_out + i, v);
+            float v = load_in1(i);
+            if (p.x_add != nullptr) v = v + p.x_add[i];
+            if (writes_sum) p.x_out[i] = v;
             ss = fmaf(v, v, ss);
         }
         ss = block_sum(ss, red);
         const float rs = 1.0f / sqrtf(ss / (float)K + p.eps);
         for (int i = tid; i < K; i += kGemvThreads) {
-            float v = act_load1<kDevLoad>(p.x + i);
-            if (p.x_add != nullptr) v = v + act_load1<kDevLoad>(p.x_add + i);
+            float v = load_in1(i);
+            if (p.x_add != nullptr) v = v + p.x_add[i];
             xs[i] = (XT)as_f32((v * rs) * p.norm_w[i]);
         }
     } else {
         for (int base = 0; base < n4; base += kGemvPrologueVecs * kGemvThreads) {
             float4_t xv[kGemvPrologueVecs], av[kGemvPrologueVecs];
 #pragma unroll
-            for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(xv[j], x4 + min(base + tid + j * kGemvThreads, n4 - 1));
+            for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = load_in4(min(base + tid + j * kGemvThreads, n4 - 1));
             if (a4 != nullptr) {
 #pragma unroll
-                for (int j = 0; j < kGemvPrologueVecs; j++) act_issue4<kDevLoad>(av[j], a4 + min(base + tid + j * kGemvThreads, n4 - 1));
-            }
-            act_wait<kDevLoad>(xv);
-            if (a4 != nullptr) {
-                act_wait<kDevLoad>(av);
+                for (int j = 0; j < kGemvPrologueVecs; j++) av[j] = a4[min(base + tid + j * kGemvThreads, n4 - 1)];
 #pragma unroll
                 for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + av[j];
             }
@@ -332,7 +313,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
             for (int j = 0; j < kGemvPrologueVecs; j++) {
                 const int i = base + tid + j * kGemvThreads;
                 if (i < n4) {
-                    if (writes_sum) act_store4<kDev>(o4 + i, xv[j]);
+                    if (writes_sum) o4[i] = xv[j];
 #pragma unroll
                     for (int e = 0; e < 4; e++) xs[i * 4 + e] = (XT)xv[j][e];
                 }
@@ -349,12 +330,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     const int n_units = p.n_rows / kRows; // n_rows is a multiple of kRows (checked on the host)
     const int W = gridDim.x * kGemvWaves;
     float acc[kMats][kRows];
-    auto clear_acc = [&]() {
-#pragma unroll
-        for (int m = 0; m < kMats; m++)
-#pragma unroll
-            for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
-    };
+    [[maybe_unused]] GreedyBest gb{-INFINITY, -1, 0}; // kArgmax: this wavefront's candidate (meaningful in lane 63)
     // the loads of the burst that starts at piece c of row unit `unit`
     auto fetch = [&](int unit, int c, uint4_t (&wv)[kU][kMats][kRows]) {
         const int row0 = unit * kRows;
@@ -394,15 +370,6 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
             }
         }
     };
-    auto take_pre = [&](auto dc, uint4_t (&wv)[kU][kMats][kRows]) {
-        constexpr int d = decltype(dc)::value;
-#pragma unroll
-        for (int u = 0; u < kU; u++)
-#pragma unroll
-            for (int m = 0; m < kMats; m++)
-#pragma unroll
-                for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[d][(u * kMats + m) * kRows + r];
-    };
     // products of one burst against x from LDS
     auto mac = [&](int c, const uint4_t (&wv)[kU][kMats][kRows]) {
 #pragma unroll
@@ -435,15 +402,19 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
             }
         if (lane == 63) {
             if constexpr (kEpi == kEpiStore) {
-                act_store1<kDev>(p.y + row0, v[0][0]);
+                p.y[row0] = v[0][0];
+            } else if constexpr (kArgmax) {
+                // the logits also go to memory; stored at device scope, because the workgroup that draws the last ticket may
+                // read them back in this same launch (see the end of this function)
+                __hip_atomic_store(p.y + row0, v[0][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                greedy_consider(gb, v[0][0], row0); // a wavefront's rows ascend, so equal values keep the lowest id
             } else if constexpr (kEpi == kEpiSilu) {
                 const float g = v[0][0];
                 const float u = v[1][0];
                 const float sg = g / (1.0f + expf(-g)); // tensor.rs:826-827
                 const float mval = sg * u;              // tensor.rs:729
-                act_store1<kDev>(p.y + row0, p.x_f16 ? f16r(mval) : mval); // transformer.rs:563-565 (cast to w2's dtype)
+                p.y[row0] = p.x_f16 ? f16r(mval) : mval; // transformer.rs:563-565 (cast to w2's dtype)
             } else { // kEpiRopeKv: rows [0, dim) = wq, [dim, 2 dim) = wk, [2 dim, 3 dim) = wv
-                // q and the cache rows are read by the attention kernel, a later launch: ordinary stores
                 const int which = row0 / p.dim;
                 const int jdx = row0 - which * p.dim;
                 const int head = jdx / p.head_dim;
@@ -473,46 +444,121 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
         }
     };
 
-    if constexpr (kPre == kPreGiven) {
-        // The wavefront's bursts as one sequence, the first kD of them possibly already in registers (gemv_issue_bursts walks
-        // the same sequence).
-        int unit = unit_first, c = 0;
-        clear_acc();
-        auto advance = [&]() {
-            c += kU;
-            if (c >= pieces) {
-                finish(unit);
-                clear_acc();
-                c = 0;
-                unit += W;
-            }
-        };
-        static_for<kD>([&](auto dc) {
-            constexpr int d = decltype(dc)::value;
-            if (unit < n_units) {
-                uint4_t wv[kU][kMats][kRows];
-                if (pre_mask & (1u << d)) take_pre(dc, wv);
-                else fetch(unit, c, wv);
-                mac(c, wv);
-                advance();
-            }
-        });
-        while (unit < n_units) {
+    for (int unit = unit_first; unit < n_units; unit += W) {
+#pragma unroll
+        for (int m = 0; m < kMats; m++)
+#pragma unroll
+            for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
+        for (int c = 0; c < pieces; c += kU) {
             uint4_t wv[kU][kMats][kRows];
-            fetch(unit, c, wv);
-            mac(c, wv);
-            advance();
-        }
-    } else {
-        for (int unit = unit_first; unit < n_units; unit += W) {
-            clear_acc();
-            for (int c = 0; c < pieces; c += kU) {
-                uint4_t wv[kU][kMats][kRows];
-                if (kPre != kPreNone && (pre_mask & 1u) && c == 0 && unit == unit_first) take_pre(std::integral_constant<int, 0>{}, wv);
-                else fetch(unit, c, wv);
-                mac(c, wv);
+            if (kPre != kPreNone && have_pre && c == 0 && unit == unit_first) {
+#pragma unroll
+                for (int u = 0; u < kU; u++)
+#pragma unroll
+                    for (int m = 0; m < kMats; m++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[(u * kMats + m) * kRows + r];
+            } else {
+                fetch(unit, c, wv);
             }
-            finish(unit);
+            mac(c, wv);
+        }
+        finish(unit);
+    }
+
+    if constexpr (kArgmax) {
+        // ---- the greedy pick over all rows (TokenSampler::sample at top_k = 1, token_sampler.rs:99-147, as
+        //      argmax_advance_kernel runs it at temperature 1) without a launch of its own ----
+        // Every workgroup reduces its wavefronts' candidates and publishes one (value, id, NaN seen) record; the workgroup
+        // that draws the last ticket reduces the records and advances the token-step state.  The hand-over uses device-scope
+        // (write-through) stores that are waited for before the ticket is drawn, and device-scope loads after it.  That a
+        // store acknowledged to the wavefront (vmcnt) is visible to a later device-scope load from another compute unit is a
+        // property of this part (gfx950: device-scope stores write through the XCD's L2 to memory, device-scope loads miss
+        // it), not a guarantee of the HIP memory model for relaxed atomics; rlh_init refuses every other architecture.
+        __shared__ float am_val[kGemvWaves];
+        __shared__ int am_idx[kGemvWaves];
+        __shared__ int am_nan[kGemvWaves];
+        __shared__ int am_last;
+        if (lane == 63) {
+            am_val[wave] = gb.best;
+            am_idx[wave] = gb.idx;
+            am_nan[wave] = gb.nan;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            GreedyBest b{am_val[0], am_idx[0], am_nan[0]};
+#pragma unroll
+            for (int w = 1; w < kGemvWaves; w++) greedy_merge(b, am_val[w], am_idx[w], am_nan[w]);
+            float *rec = p.amax_ws + (size_t)blockIdx.x * 4;
+            __hip_atomic_store(rec + 0, b.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(reinterpret_cast<int *>(rec) + 1, b.idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(reinterpret_cast<int *>(rec) + 2, b.nan, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // every store of this workgroup (its logits and its record) has been acknowledged before its ticket is drawn
+        asm volatile("" ::: "memory");
+        wait_vmcnt<0>();
+        asm volatile("" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned prev = __hip_atomic_fetch_add(p.amax_ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = prev == gridDim.x - 1;
+            if (last) __hip_atomic_store(p.amax_ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
+            am_last = last;
+        }
+        __syncthreads();
+        if (!am_last) return;
+        GreedyBest b{-INFINITY, -1, 0};
+        for (int blk = tid; blk < (int)gridDim.x; blk += kGemvThreads) { // ascending ids per thread: ties keep the lowest id
+            const float *rec = p.amax_ws + (size_t)blk * 4;
+            const float ov = __hip_atomic_load(rec + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int oi = __hip_atomic_load(reinterpret_cast<const int *>(rec) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int on = __hip_atomic_load(reinterpret_cast<const int *>(rec) + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            greedy_merge(b, ov, oi, on);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(b.best, off, kWave);
+            const int oi = __shfl_xor(b.idx, off, kWave);
+            const int on = __shfl_xor(b.nan, off, kWave);
+            greedy_merge(b, ov, oi, on);
+        }
+        __syncthreads(); // am_* are about to be reused
+        if (lane == 0) {
+            am_val[wave] = b.best;
+            am_idx[wave] = b.idx;
+            am_nan[wave] = b.nan;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < kGemvWaves; w++) greedy_merge(b, am_val[w], am_idx[w], am_nan[w]); // every thread ends with the grid's pick
+        // Can sum(exp(l)) overflow f32?  Only if vocab * exp(largest) can: largest > ln(FLT_MAX) - ln(vocab).  Then (rare) the
+        // sum decides, formed in double over the stored logits like argmax_advance_kernel does.
+        const float kLnFltMax = 88.72283172607422f;
+        const bool sum_at_risk = !b.nan && b.best <= kLnFltMax && b.best > kLnFltMax - logf((float)p.n_rows);
+        double total = 0.0;
+        if (sum_at_risk) { // uniform over the workgroup
+            __shared__ double am_sum[kGemvWaves];
+            double part = 0.0;
+            for (int i = tid; i < p.n_rows; i += kGemvThreads) {
+                const float v = i == 0 ? 0.0f : __hip_atomic_load(p.y + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                part += exp((double)v);
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) part += __shfl_xor(part, off, kWave);
+            if (lane == 0) am_sum[wave] = part;
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < kGemvWaves; w++) total += am_sum[w];
+        }
+        if (tid == 0) {
+            int pick = b.idx < 0 ? 0 : b.idx;                                                   // every logit NaN
+            if (b.nan || b.best > kLnFltMax || total > 3.4028234663852886e38) pick = 0;        // sum not finite: every probability 0 or NaN
+            DecodeState *st = p.state_rw;
+            st->token = pick;
+            st->pos = st->pos + 1;
+            const int k = st->n_out;
+            if (p.out_tokens != nullptr && k < p.out_cap) p.out_tokens[k] = pick;
+            st->n_out = k + 1;
         }
     }
 }

@@ -10,7 +10,10 @@ namespace rlh {
 enum GemvEpilogue {
     kEpiStore = 0,   // y[c] = v
     kEpiRopeKv = 2,  // fused wq|wk|wv: RoPE on q and k, q -> y, k/v -> KV cache at *pos
-    kEpiSilu = 3     // two matrices (w1, w3): y[c] = silu(v1) * v3   (transformer.rs:561-562)
+    kEpiSilu = 3,    // two matrices (w1, w3): y[c] = silu(v1) * v3   (transformer.rs:561-562)
+    kEpiStoreArgmax = 4 // y[c] = v, and the greedy pick over all rows (TokenSampler::sample at top_k = 1, temperature 1) in the same
+                     // launch: the last workgroup to finish reduces the workgroups' candidates and advances the token-step
+                     // state like argmax_advance_kernel (fp32 x only)
 };
 
 // Device-resident scalars of the token loop.  Kernels read them from memory so that a recorded
@@ -38,8 +41,11 @@ struct GemvParams {
     int x_f16;                // 1: x (after the optional norm) is rounded to f16 before the product
     int round_y;              // 1: product rounded to f16 precision (tensor.rs:1623-1643)
     int stream_weights;       // 1: non-temporal weight loads
-    int rows_per_wave;        // set by launch_gemv
+    int burst_fixed;          // 1: bursts of 8 loads whatever the row length (default: a length that divides the row where one is built)
     // kEpiRopeKv only
+    const void *embed_table;  // optional [vocab x k], f16 or f32: the input row is row state->token of this table, widened to f32
+                              // (x is then unused; x_out, if set, receives the row)
+    int embed_f16;
     const DecodeState *state;
     int pos1_host;            // position + 1 where the host knows it (spares the kernel a dependent load), 0: read state->pos
     const float2 *freqs;      // [max_seq_len x head_dim/2] (cos, sin) as f32
@@ -49,30 +55,19 @@ struct GemvParams {
     int dim;
     int head_dim;
     int max_seq_len;
+    // kEpiStoreArgmax only
+    float *amax_ws;           // one 16-byte record per workgroup of the launch (gemv_argmax_ws_bytes)
+    unsigned *amax_ticket;    // arrival counter, zero before the launch; the kernel leaves it zero
+    DecodeState *state_rw;    // receives the pick: token = id, pos += 1, n_out += 1
+    int32_t *out_tokens;      // optional: out_tokens[n_out] = id while n_out < out_cap
+    int out_cap;
 };
 
 hipError_t launch_gemv(const GemvParams &p, int epilogue, hipStream_t s);
 // bytes of dynamic LDS launch_gemv will request for a given k (for capability checks)
 size_t gemv_lds_bytes(int k, int w_is_f16, int x_f16);
-
-// ---- the matrix-vector phases of one transformer block as one launch (decode_fused.hip) ----
-constexpr int kFusedGroups = 16; // arrival counters of the first barrier level
-// Barrier words in device memory, zero when created: kFusedGroups group counters, the top counter, the generation word and
-// the error word, each on its own 128-byte line.
-struct FusedBarrierState {
-    unsigned words[(kFusedGroups + 3) * 32];
-};
-struct FusedLayerParams {
-    GemvParams wo, w13, w2; // kEpiStore, kEpiSilu, kEpiStore
-    GemvParams last;        // what follows w2: the next block's wq|wk|wv (kEpiRopeKv) or the output head (kEpiStore, fp32 x)
-    int last_kind;          // 0: wq|wk|wv, 1: head with f16 weights, 2: head with f32 weights
-    int n_phases;           // 4, or 3 to stop after w2
-    FusedBarrierState *barrier;
-    long long limit_ticks;  // bound of every barrier wait in 100 MHz wall-clock ticks
-};
-// blocks_out: the grid to launch with (all of it must be resident at once; bounded by the device's capacity)
-hipError_t fused_layer_grid(const FusedLayerParams &p, int compute_units, int *blocks_out);
-hipError_t launch_fused_layer(const FusedLayerParams &p, int blocks, hipStream_t s);
+// bytes of GemvParams::amax_ws that any launch can need
+size_t gemv_argmax_ws_bytes();
 
 struct AttnDecodeParams {
     const float *q;           // [n_heads x head_dim] f32 (after RoPE)
@@ -90,8 +85,8 @@ struct AttnDecodeParams {
     float *workspace;         // [n_heads x n_splits x (head_dim + 2)] partial (max, sum, weighted V), needed when n_splits > 1
     unsigned *tickets;        // [n_heads] arrival counters, needed when n_splits > 1 and the merge runs inside the kernel;
                               // zero before the launch, and the kernel leaves them zero
-    int merge_mode;           // 0: a second small kernel merges the partial results; 1 / 2: the last block of a head to finish
-                              // merges them (1: device-scope fences around the ticket, 2: device-scope stores and loads)
+    int merge_mode;           // 0: a second small kernel merges the partial results; 2: the last block of a head to finish
+                              // merges them (partial results stored and loaded at device scope)
     int chunk_hint;           // upper bound of the positions one block covers (sizes the loads in flight); 0 = unknown
     int lds_stage;            // 1: K / V tiles staged in LDS first (comparison variant; needs pos_host, an f16 cache, head_dim 64 / 128)
 };
@@ -122,6 +117,19 @@ enum GemmEpilogue {
     kGemmEpiRopeQkv = 4     // fast path only: the f16-rounded [m x 3 dim] product of wq|wk|wv is not stored; RoPE on its q and k
                             // columns, q as hi + lo halves, k and v into the cache, v transposed (GemmParams::rope; what
                             // rope_kv_prefill_tiled_kernel does with the stored product: transformer.rs:704-761)
+};
+
+// Switches of the prompt-path products; all zero = the launchers' own choices.  They come from the context (parsed from the
+// environment once, when the context is made; rlh_set_option changes them), never from the environment at launch time.
+struct GemmTune {
+    int tile_plus1;       // GEMM_TILE=0..3 forces the tile (128x128, 256x128, 256x192, 256x256): stored as tile + 1
+    int split_k;          // GEMM_SPLIT_K=N forces N K-pieces for the products that qualify for a cut along K
+    int no_split_half;    // GEMM_SPLIT_HALF=0: cut along K only when the tiles cover at most a quarter of the compute units
+    int dual_plus1;       // GEMM_DUAL=0..5: w1 and w3 in one pass never (0) / in that form wherever the kernel can run: stored as mode + 1
+    int no_dual_cut;      // GEMM_DUAL_CUT=0: the one-pass w1|w3 product always covers all columns
+    int no_rope_epilogue; // GEMM_ROPE=0: RoPE, q hi/lo, cache rows and V^T as a kernel of their own on the stored wq|wk|wv product
+    int no_finish_norm;   // FINISH_NORM=0: the RMSNorm after a split wo / w2 product as a kernel of its own
+    int no_kgroup;        // GEMM_KGROUP=0: 128x128 products stay on the kernel whose wavefronts split the tile
 };
 
 struct GemmParams {
@@ -156,6 +164,7 @@ struct GemmParams {
     _Float16 *norm_out;     // [m x n], row stride n
     float norm_eps;
     int *norm_done;         // host flag
+    GemmTune tune;          // the context's switches (zero = defaults)
     PrefillRopeParams rope; // kGemmEpiRopeQkv: the destinations (qkv unused; n = m, 3 dim = n, f16 cache, vt_swap as the reader expects)
 };
 
@@ -182,7 +191,6 @@ struct AttnPrefillParams {
     int n, n_heads, head_dim, dim, max_seq_len, t_pad;
     float scale;             // 1 / sqrt(head_dim) (transformer.rs:770)
     int order;               // launch order of the query blocks: 0 ascending, 1 descending, 2 descending then ascending
-    int key_parts;           // 2 (or 0): four wavefronts on 64-key tiles, t_pad % 64 == 0; 4: eight wavefronts on 128-key tiles, t_pad % 128 == 0
 };
 bool attn_prefill_supported(int head_dim);
 hipError_t launch_attn_prefill(const AttnPrefillParams &p, hipStream_t s);

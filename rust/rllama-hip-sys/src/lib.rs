@@ -85,6 +85,7 @@ extern "C" {
     pub fn rlh_shutdown(ctx: *mut rlh_ctx);
     pub fn rlh_sync(ctx: *mut rlh_ctx) -> c_int;
     pub fn rlh_last_error() -> *const c_char;
+    pub fn rlh_set_option(ctx: *mut rlh_ctx, name: *const c_char, value: *const c_char) -> c_int;
     pub fn rlh_device_info(ctx: *mut rlh_ctx, name: *mut c_char, cap: c_int, compute_units: *mut c_int, hbm_bytes: *mut u64) -> c_int;
     pub fn rlh_model_create(ctx: *mut rlh_ctx, params: *const rlh_model_params, out: *mut *mut rlh_model) -> c_int;
     pub fn rlh_model_free(model: *mut rlh_model);

@@ -2,6 +2,8 @@
 and an independent float64 LLaMA forward (library matmuls, textbook formulas) that pins the oracle."""
 from __future__ import annotations
 
+import contextlib
+
 import numpy as np
 
 import oracle
@@ -81,6 +83,19 @@ def make_gpu(ctx, shape: Shape, W, force_f16: bool) -> rllama_amd.Transformer:
     return m
 
 
+@contextlib.contextmanager
+def options(ctx, **switches):
+    """Sets switches of the library on the context (rlh_set_option: NAME of the RLLAMA_HIP_<NAME> variables) for the
+    duration of a with block, then puts the defaults back."""
+    try:
+        for name, value in switches.items():
+            ctx.set_option(name, value)
+        yield
+    finally:
+        for name in switches:
+            ctx.set_option(name, None)
+
+
 def to_f64(arr: np.ndarray) -> np.ndarray:
     if arr.dtype == np.uint16:
         return arr.view(np.float16).astype(np.float64)
@@ -100,8 +115,9 @@ def max_rel_err(a: np.ndarray, b: np.ndarray) -> float:
 # with numpy's matmul and float16 casts -- none of the oracle's loops or lane orders.
 # ---------------------------------------------------------------------------------------------------------
 class RefF64:
-    def __init__(self, shape: Shape, W, f16_points: bool):
+    def __init__(self, shape: Shape, W, f16_points: bool, via_f32: bool = False):
         self.s = shape
+        self.via_f32 = via_f32   # round to f32 first, then to f16: the reference's values are f32 before every cast
         self.W = {k: to_f64(v) for k, v in W.items()}
         self.f16_points = f16_points
         L, H, hd, T = shape.n_layers, shape.n_heads, shape.head_dim, shape.max_seq_len
@@ -109,7 +125,11 @@ class RefF64:
         self.v = np.zeros((L, H, T, hd))
 
     def r(self, x):
-        return x.astype(np.float16).astype(np.float64) if self.f16_points else x
+        if not self.f16_points:
+            return x
+        if self.via_f32:
+            return x.astype(np.float32).astype(np.float16).astype(np.float64)
+        return x.astype(np.float16).astype(np.float64)
 
     def norm(self, x, w):
         return x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + self.s.norm_eps) * w
@@ -154,18 +174,18 @@ class RefF64:
         return xf[-1] @ W[(OUTPUT, 0)].T
 
 
-def oracle_from_device(gm: "rllama_amd.Transformer", max_seq_len: int) -> oracle.Model:
-    """An oracle model holding exactly the bits the device model holds (f16 mode): every tensor is read back from HBM and
-    handed to the oracle, so both sides start from the same weights whatever filled them."""
+def oracle_from_device(gm: "rllama_amd.Transformer", max_seq_len: int, force_f16: bool = True) -> oracle.Model:
+    """An oracle model holding exactly the values the device model holds: every tensor is read back from HBM and handed to
+    the oracle (f16 bits in f16 mode, fp32 values in f32 mode), so both sides start from the same weights whatever filled them."""
     d, L, H, F, V = gm.dim, gm.n_layers, gm.n_heads, gm.ffn_hidden, gm.vocab_size
-    om = oracle.Model(d, L, H, F, V, max_seq_len, gm.params.norm_eps, True)
+    om = oracle.Model(d, L, H, F, V, max_seq_len, gm.params.norm_eps, force_f16)
     shapes = {WQ: (d, d), WK: (d, d), WV: (d, d), WO: (d, d), W1: (F, d), W3: (F, d), W2: (d, F)}
     for kind in (TOK_EMB, OUTPUT):
-        om.set_tensor(kind, 0, gm.get_tensor(kind, 0, V, d, as_f16_bits=True))
+        om.set_tensor(kind, 0, gm.get_tensor(kind, 0, V, d, as_f16_bits=True))   # held as f16 on the device in both modes (exact)
     om.set_tensor(NORM, 0, gm.get_tensor(NORM, 0, 1, d))
     for l in range(L):
         for kind, (r, c) in shapes.items():
-            om.set_tensor(kind, l, gm.get_tensor(kind, l, r, c, as_f16_bits=True))
+            om.set_tensor(kind, l, gm.get_tensor(kind, l, r, c, as_f16_bits=force_f16))
         for kind in (ATTN_NORM, FFN_NORM):
             om.set_tensor(kind, l, gm.get_tensor(kind, l, 1, d))
     return om

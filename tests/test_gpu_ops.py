@@ -12,6 +12,7 @@ import pytest
 import oracle
 import rllama_amd
 from rllama_amd import Tensor, TensorDType
+from common import options
 
 pytestmark = pytest.mark.gpu
 f32 = np.float32
@@ -191,14 +192,10 @@ def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
     want = (silu * u).astype(np.float16)
     X, W1, W3 = Tensor.from_numpy(ctx, x), Tensor.from_numpy(ctx, w1), Tensor.from_numpy(ctx, w3)
     got = {}
-    os.environ["RLLAMA_HIP_GEMM_KGROUP"] = "0"  # the two-launch form on the kernel whose sum over k runs in the one-pass kernel's order
     for mode in ("1", "2", "3", "4", "5", "0"):  # five shapes of the one-pass workgroup, two launches
-        os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
-        try:
+        # (GEMM_KGROUP=0: the two-launch form on the kernel whose sum over k runs in the one-pass kernel's order)
+        with options(ctx, GEMM_KGROUP="0", GEMM_DUAL=mode):
             got[mode] = X.ffn_gate(W1, W3).to_numpy()
-        finally:
-            del os.environ["RLLAMA_HIP_GEMM_DUAL"]
-    del os.environ["RLLAMA_HIP_GEMM_KGROUP"]
     assert np.array_equal(got["1"].view(np.uint16), got["0"].view(np.uint16))
     for mode in ("2", "3", "4", "5"):
         assert np.array_equal(got[mode].view(np.uint16), got["0"].view(np.uint16)), mode
@@ -211,7 +208,7 @@ def test_ffn_gate_against_the_reference_ops(ctx, n, m, k):
         Tensor.from_numpy(ctx, x.astype(f32)).ffn_gate(W1, W3)                                       # f16 mode only
 
 
-def test_ffn_gate_whole_rounds_in_one_pass_and_the_rest_in_two_launches(ctx, monkeypatch):
+def test_ffn_gate_whole_rounds_in_one_pass_and_the_rest_in_two_launches(ctx):
     """2048 rows x 13824 columns are 576 workgroups of the one-pass form, 2.25 rounds of the 256 compute units: the pass takes
     the 12288 columns that make two whole rounds and the last 1536 go through w1's product and w3's with the gate epilogue
     (src/transformer.rs:551-565 either way).  Against the two-launch form over all columns (a few f16 steps apart on few
@@ -224,11 +221,9 @@ def test_ffn_gate_whole_rounds_in_one_pass_and_the_rest_in_two_launches(ctx, mon
     w1 = (rng.standard_normal((m, k)) * 0.05).astype(np.float16)
     w3 = (rng.standard_normal((m, k)) * 0.05).astype(np.float16)
     X, W1, W3 = Tensor.from_numpy(ctx, x), Tensor.from_numpy(ctx, w1), Tensor.from_numpy(ctx, w3)
-    monkeypatch.delenv("RLLAMA_HIP_GEMM_DUAL", raising=False)
     got = X.ffn_gate(W1, W3).to_numpy()
-    monkeypatch.setenv("RLLAMA_HIP_GEMM_DUAL", "0")
-    two = X.ffn_gate(W1, W3).to_numpy()
-    monkeypatch.delenv("RLLAMA_HIP_GEMM_DUAL")
+    with options(ctx, GEMM_DUAL="0"):
+        two = X.ffn_gate(W1, W3).to_numpy()
     step = np.spacing(np.maximum(np.abs(got), np.abs(two))).astype(f32)
     assert np.array_equal(got[:, :12288], two[:, :12288])   # the pass: the two-launch form's order of additions
     assert np.mean(got[:, 12288:] != two[:, 12288:]) < 5e-3 and np.all(np.abs(got.astype(f32) - two.astype(f32)) <= 8 * step)
@@ -242,14 +237,11 @@ def test_ffn_gate_whole_rounds_in_one_pass_and_the_rest_in_two_launches(ctx, mon
     assert np.all(np.abs(have - want) <= 4e-3 * np.abs(want) + 1e-4), float(np.max(np.abs(have - want)))
 
 
-@pytest.mark.parametrize("parts", [2, 4])
 @pytest.mark.parametrize("hd,H,n", [(128, 2, 200), (64, 3, 65), (128, 1, 64), (64, 2, 1), (128, 2, 333)])
-def test_attn_prefill_against_the_reference_ops(ctx, hd, H, n, parts, monkeypatch):
+def test_attn_prefill_against_the_reference_ops(ctx, hd, H, n):
     """The prompt's attention block between the projections and wo against the oracle's restatement of
     src/transformer.rs:704-796: RoPE, f16 cache rows, per row scores by the sequential-k product (src/tensor.rs:1050-1115),
-    mask, softmax, P.V by dot8, heads concatenated and rounded to f16.  Ragged query / key tiles included; both forms of the
-    kernel (four wavefronts on 64-key tiles, eight on 128-key tiles)."""
-    monkeypatch.setenv("RLLAMA_HIP_PREFILL_ATTN_PARTS", str(parts))
+    mask, softmax, P.V by dot8, heads concatenated and rounded to f16.  Ragged query / key tiles included."""
     rng = np.random.default_rng(hd + H * 13 + n)
     d, S = H * hd, 352
     qkv = (rng.standard_normal((n, 3 * d)) * 0.8).astype(np.float16)
@@ -318,6 +310,44 @@ def test_device_greedy_pick_on_crafted_logits(ctx, name, temperature):
     sampler = rllama_amd.TokenSampler().temperature(temperature).top_k(1).top_p(1.0).repetition_penalty(1.0)
     host, _ = sampler.sample(logits, [], np.random.default_rng(0))
     assert host == want, (name, temperature, host, want)
+
+
+@pytest.mark.parametrize("name", sorted(_greedy_cases()))
+def test_greedy_pick_inside_the_output_head_on_crafted_logits(ctx, name):
+    """The pick that a decode step makes inside the output head's launch, on the same crafted cases: a one-layer f32-mode model
+    whose wo and w2 are zero and whose embedding rows all hold one non-zero element, so that every step's logits are
+    W_out[:, 0] times one constant -- the crafted values.  The second id of a greedy run comes from a decode step; it must
+    be what the oracle's sampler picks on the logits the device itself returns."""
+    from rllama_amd import ATTN_NORM, FFN_NORM, NORM, OUTPUT, TOK_EMB, W1, W2, W3, WK, WO, WQ, WV
+    logits = _greedy_cases()[name]
+    V, d, F = logits.size, 64, 64
+    gm = rllama_amd.Transformer(ctx, d, 1, 2, F, V, 8, 1e-6, rllama_amd.DataSettings(ctx))
+    rng = np.random.default_rng(3)
+    emb = np.zeros((V, d), f32)
+    emb[:, 0] = 8.0                                         # mean(x^2) = 1: the final norm leaves 8 / sqrt(1 + eps) in element 0
+    xn0 = f32(8.0) * (f32(1.0) / np.sqrt(f32(1.0) + f32(1e-6)))
+    out = np.zeros((V, d), f32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        out[:, 0] = logits / xn0
+    gm.set_tensor(TOK_EMB, 0, emb)
+    gm.set_tensor(OUTPUT, 0, out)
+    gm.set_tensor(NORM, 0, np.ones((1, d), f32))
+    for kind, shape in ((WQ, (d, d)), (WK, (d, d)), (WV, (d, d)), (W1, (F, d)), (W3, (F, d))):
+        gm.set_tensor(kind, 0, (rng.standard_normal(shape) * 0.1).astype(f32))
+    gm.set_tensor(WO, 0, np.zeros((d, d), f32))
+    gm.set_tensor(W2, 0, np.zeros((d, F), f32))
+    for kind in (ATTN_NORM, FFN_NORM):
+        gm.set_tensor(kind, 0, np.ones((1, d), f32))
+    have = gm.forward([5], 0, gm.make_caches())
+    finite = np.isfinite(logits)
+    assert np.allclose(have[finite], logits[finite], rtol=1e-6, atol=1e-6) and np.array_equal(np.isnan(have), np.isnan(logits))
+    want, _, _ = oracle.sample_greedy(have, 1.0)
+    ids, _, _ = gm.generate_greedy([5], 3, gm.make_caches())
+    assert ids.tolist() == [want, want, want], (name, ids.tolist(), want)   # the prompt pass's pick, then two decode steps
+    with options(ctx, DECODE_FOLD="0"):
+        ids2, _, _ = gm.generate_greedy([5], 3, gm.make_caches())
+    assert ids2.tolist() == ids.tolist()
+    gm.free()
 
 
 def test_device_greedy_pick_full_vocab_and_odd_sizes(ctx):

@@ -11,7 +11,7 @@ import pytest
 import oracle
 import rllama_amd
 from rllama_amd import Tensor, TensorDType
-from common import (CONFIG0, PER_LAYER, SMALL, TINY, Shape, make_gpu, make_oracle, max_rel_err, random_f32_weights, synth_weights)
+from common import (CONFIG0, PER_LAYER, SMALL, TINY, Shape, make_gpu, make_oracle, max_rel_err, options, random_f32_weights, synth_weights)
 
 pytestmark = pytest.mark.gpu
 f32 = np.float32
@@ -84,7 +84,7 @@ def test_gemv_f16_weights(ctx, m_rows, k):
 
 
 @pytest.mark.parametrize("m_rows,k,burst", [(300, 11008, 11), (130, 5376, 11), (64, 4608, 9), (2100, 13824, 9), (77, 5120, 10), (40, 3584, 7), (9, 6656, 8)])
-def test_gemv_burst_length_follows_the_row(ctx, m_rows, k, burst, monkeypatch):
+def test_gemv_burst_length_follows_the_row(ctx, m_rows, k, burst):
     """The single-row product issues its loads in bursts of 7, 9, 10 or 11 per lane where that divides the row's pieces of 512
     halves and 8 does not (a row that ends inside a piece counts as whole pieces: 11008 -> 22, 5376 -> 11); the last case has
     13 pieces and keeps 8 with a partial last burst.  Every lane still adds its products in the order of the pieces, so the
@@ -97,9 +97,9 @@ def test_gemv_burst_length_follows_the_row(ctx, m_rows, k, burst, monkeypatch):
     W, X = Tensor.from_numpy(ctx, wh), Tensor.from_numpy(ctx, x)
     got = W.gemv(X, round_x=True, round_y=True).to_numpy()[0]
     got32 = W.gemv(X, round_x=False, round_y=False).to_numpy()[0]
-    monkeypatch.setenv("RLLAMA_HIP_GEMV_BURST", "0")
-    assert np.array_equal(got, W.gemv(X, round_x=True, round_y=True).to_numpy()[0])
-    assert np.array_equal(got32, W.gemv(X, round_x=False, round_y=False).to_numpy()[0])
+    with options(ctx, GEMV_BURST="0"):
+        assert np.array_equal(got, W.gemv(X, round_x=True, round_y=True).to_numpy()[0])
+        assert np.array_equal(got32, W.gemv(X, round_x=False, round_y=False).to_numpy()[0])
     want = oracle.f16_bits_to_f32(oracle.matmul_transposed_f16(xh, wh))[0]
     mag = np.abs(oracle.f16_bits_to_f32(xh).astype(np.float64))[0] @ np.abs(oracle.f16_bits_to_f32(wh).astype(np.float64)).T
     close_f16(got, want, mag, "gemv f16, burst length by row")
@@ -258,27 +258,25 @@ def test_prefill_fused_attention_head_dims(ctx, n_heads, n, cap):
     gm.free()
 
 
-def test_prefill_attention_gemm_form_for_large_heads(ctx, monkeypatch):
-    """RLLAMA_HIP_PREFILL_ATTN=gemm (read when a model is created) keeps head_dim 64 / 128 on the two-GEMM form of the
+def test_prefill_attention_gemm_form_for_large_heads(ctx):
+    """The PREFILL_ATTN=gemm switch keeps head_dim 64 / 128 on the two-GEMM form of the
     prefill attention (hi | lo halves of q and of P as K segments, tiles above the diagonal skipped, V^T in natural key
     order): same function as the one-kernel form and the oracle."""
     shape = Shape(dim=256, n_layers=2, n_heads=2, ffn_hidden=512, vocab_size=128, max_seq_len=320)   # head_dim 128
     W = synth_weights(shape, seed=53, std=0.08, norm_ones=False)
     toks = np.random.default_rng(54).integers(0, shape.vocab_size, 301)
     om = make_oracle(shape, W, True)
-    fused = make_gpu(ctx, shape, W, True)
-    monkeypatch.setenv("RLLAMA_HIP_PREFILL_ATTN", "gemm")
-    gemm_form = make_gpu(ctx, shape, W, True)
-    monkeypatch.delenv("RLLAMA_HIP_PREFILL_ATTN")
+    gm = make_gpu(ctx, shape, W, True)
     for n in (300, 65):
-        oc, ca, cb = om.make_caches(), fused.make_caches(), gemm_form.make_caches()
+        oc, ca, cb = om.make_caches(), gm.make_caches(), gm.make_caches()
         want = om.forward(toks[:n], 0, oc)
-        a, b = fused.forward(toks[:n], 0, ca), gemm_form.forward(toks[:n], 0, cb)
+        a = gm.forward(toks[:n], 0, ca)
+        with options(ctx, PREFILL_ATTN="gemm"):
+            b = gm.forward(toks[:n], 0, cb)
         assert max_rel_err(a, want) < TOL_F16 and max_rel_err(b, want) < TOL_F16, (n, max_rel_err(a, want), max_rel_err(b, want))
         want1 = om.forward(toks[n:n + 1], n, oc)
-        assert max_rel_err(gemm_form.forward(toks[n:n + 1], n, cb), want1) < TOL_F16
-    fused.free()
-    gemm_form.free()
+        assert max_rel_err(gm.forward(toks[n:n + 1], n, cb), want1) < TOL_F16
+    gm.free()
 
 
 def test_prefill_odd_dims_register_staged_gemm(ctx):
@@ -309,12 +307,9 @@ def test_prefill_short_prompt_split_k(ctx):
         assert max_rel_err(gm.forward(toks[n:n + 1], n, gc), om.forward(toks[n:n + 1], n, oc)) < TOL_F16
         # the kernel that adds the partial sums of wo / w2 also writes the RMSNorm that follows; with that switched off the
         # norm runs as a kernel of its own: same arithmetic in the same order, so the same bits
-        os.environ["RLLAMA_HIP_FINISH_NORM"] = "0"
-        try:
+        with options(ctx, FINISH_NORM="0"):
             g2 = gm.make_caches()
             assert np.array_equal(gm.forward(toks[:n], 0, g2), got)
-        finally:
-            del os.environ["RLLAMA_HIP_FINISH_NORM"]
     gm.free()
 
 
@@ -332,7 +327,7 @@ def test_prefill_wide_ffn_largest_tile(ctx):
 
 
 @pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 1000, 300), (128, 2, 192, 256), (192, 3, 1544, 515)])
-def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n, monkeypatch):
+def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n):
     """w1 and w3 as one pass over the normalised rows (two accumulator sets per wavefront, SiLU(w1 x) * (w3 x) straight from
     them: transformer.rs:551-565), forced onto shapes the oracle handles quickly: ragged last row and column tiles (300 and
     515 rows on 256-row tiles, 1000 = 5 x 192 + 40 and 1544 = 8 x 192 + 8 columns), exactly one tile, three K-tiles.  Same
@@ -342,16 +337,12 @@ def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n, monkeypatch):
     toks = np.random.default_rng(62).integers(0, shape.vocab_size, n + 1)
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
     got = {}
-    # (the two-launch form on the tile-splitting kernel, whose sum over k runs in the same order as the one-pass kernel's)
-    monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", "0")
     # workgroups of 256 x 192 of both products (eight wavefronts), 128 x 192 (four), the short-prompt forms 32 / 64 / 128 x 64, two launches
+    # (GEMM_KGROUP=0: the two-launch form on the tile-splitting kernel, whose sum over k runs in the same order as the one-pass kernel's)
     for mode in ("1", "2", "3", "4", "5", "0"):
-        os.environ["RLLAMA_HIP_GEMM_DUAL"] = mode
-        try:
+        with options(ctx, GEMM_KGROUP="0", GEMM_DUAL=mode):
             gc = gm.make_caches()
             got[mode] = (gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc))
-        finally:
-            del os.environ["RLLAMA_HIP_GEMM_DUAL"]
     for mode in ("1", "2", "3", "4", "5"):
         assert np.array_equal(got[mode][0], got["0"][0]) and np.array_equal(got[mode][1], got["0"][1]), mode
     oc = om.make_caches()
@@ -361,7 +352,7 @@ def test_prefill_w1_w3_in_one_pass(ctx, dim, heads, ffn, n, monkeypatch):
 
 
 @pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 384, 300), (128, 2, 256, 70), (64, 4, 128, 130), (192, 3, 256, 515), (512, 4, 640, 1024)])
-def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n, monkeypatch):
+def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n):
     """RoPE, the hi + lo halves of q, the cache rows and V^T written by the epilogue of the wq|wk|wv product (transformer.rs:
     694-761 with seq_len > 1) against the same steps as a kernel of their own on the stored product: same values at the
     same rounding points, so the same bits in the logits, in the token step that follows, and in every cache row.  Head
@@ -372,16 +363,12 @@ def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n,
     toks = np.random.default_rng(72).integers(0, shape.vocab_size, n + 1)
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
     got = {}
-    # (the stored product on the tile-splitting kernel, whose sum over k runs in the same order as the kernel with the epilogue)
-    monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", "0")
+    # (GEMM_KGROUP=0: the stored product on the tile-splitting kernel, whose sum over k runs in the same order as the kernel with the epilogue)
     for mode in ("1", "0"):
-        os.environ["RLLAMA_HIP_GEMM_ROPE"] = mode
-        try:
+        with options(ctx, GEMM_KGROUP="0", GEMM_ROPE=mode):
             gc = gm.make_caches()
             a, b = gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc)
             got[mode] = (a, b, [gc.read(l, h, w) for l in range(2) for h in range(heads) for w in (0, 1)])
-        finally:
-            del os.environ["RLLAMA_HIP_GEMM_ROPE"]
     assert np.array_equal(got["1"][0], got["0"][0]) and np.array_equal(got["1"][1], got["0"][1])
     for x, y in zip(got["1"][2], got["0"][2]):
         assert np.array_equal(x, y)
@@ -392,7 +379,7 @@ def test_prefill_rope_and_cache_write_in_the_projection(ctx, dim, heads, ffn, n,
 
 
 @pytest.mark.parametrize("dim,heads,ffn,n", [(256, 2, 704, 300), (512, 4, 1408, 520), (128, 2, 192, 130)])
-def test_prefill_k_steps_split_among_wavefronts(ctx, dim, heads, ffn, n, monkeypatch):
+def test_prefill_k_steps_split_among_wavefronts(ctx, dim, heads, ffn, n):
     """wo and w2 (and the other projections at these sizes) on the kernel whose wavefronts split the K-steps of a 128 x 128 tile
     and add their four partial sums through LDS: against the oracle, and close to the tile-splitting kernel (the order of the
     fp32 additions differs, so single f16 rounding decisions may)."""
@@ -402,9 +389,9 @@ def test_prefill_k_steps_split_among_wavefronts(ctx, dim, heads, ffn, n, monkeyp
     om, gm = make_oracle(shape, W, True), make_gpu(ctx, shape, W, True)
     got = {}
     for mode in ("1", "0"):
-        monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", mode)
-        gc = gm.make_caches()
-        got[mode] = (gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc))
+        with options(ctx, GEMM_KGROUP=mode):
+            gc = gm.make_caches()
+            got[mode] = (gm.forward(toks[:n], 0, gc), gm.forward(toks[n:n + 1], n, gc))
     oc = om.make_caches()
     want = (om.forward(toks[:n], 0, oc), om.forward(toks[n:n + 1], n, oc))
     for i in (0, 1):
@@ -790,16 +777,16 @@ def test_layer_span_on_a_whole_model_equals_its_forward(ctx):
 @pytest.mark.parametrize("n,m_rows,k", [(2, 3, 8), (33, 65, 72), (128, 128, 64), (130, 200, 192), (16, 2816, 1024), (257, 384, 4096), (1024, 256, 11008),
                                         (1024, 12288, 64), (1000, 12290, 160), (1024, 16384, 96), (512, 16384, 96)])
 @pytest.mark.parametrize("kgroup", ["1", "0"], ids=["k-steps-split", "tile-split"])
-def test_mfma_gemm_f16(ctx, n, m_rows, k, kgroup, monkeypatch):
+def test_mfma_gemm_f16(ctx, n, m_rows, k, kgroup):
     """src [n x k] . other[m x k]^T with n > 1 runs on the matrix cores; every element against the oracle's
     f16-rounded dot8 (tensor.rs:1476-1666), including tiles that straddle the matrix edges.  Products that take 128 x 128
     tiles with k a multiple of 64 run on the kernel whose wavefronts split the K-steps of a tile (four partial sums per
     element, added in a fixed order) unless that is switched off; both forms are checked."""
-    monkeypatch.setenv("RLLAMA_HIP_GEMM_KGROUP", kgroup)
     rng = np.random.default_rng(n * 7 + m_rows * 3 + k)
     a = oracle.f32_to_f16_bits(rng.uniform(-1, 1, (n, k)).astype(f32))
     b = oracle.f32_to_f16_bits((rng.standard_normal((m_rows, k)) * 0.05).astype(f32))
-    got = Tensor.from_numpy(ctx, a).matrix_mul_transposed(Tensor.from_numpy(ctx, b)).to_numpy().astype(f32)
+    with options(ctx, GEMM_KGROUP=kgroup):
+        got = Tensor.from_numpy(ctx, a).matrix_mul_transposed(Tensor.from_numpy(ctx, b)).to_numpy().astype(f32)
     want = oracle.f16_bits_to_f32(oracle.matmul_transposed_f16(a, b))
     mag = np.abs(oracle.f16_bits_to_f32(a).astype(np.float64)) @ np.abs(oracle.f16_bits_to_f32(b).astype(np.float64)).T
     close_f16(got, want, mag, f"mfma gemm {n}x{m_rows}x{k}")
@@ -881,31 +868,57 @@ def test_prefill_matrix_core_path_against_token_by_token_and_oracle(ctx):
     gm.free()
 
 
-def test_decode_step_graph_replay(ctx, monkeypatch):
-    """RLLAMA_HIP_DECODE_GRAPH=1 replays the captured decode step (one graph per attention grid shape): the ids are those of
+def test_decode_step_graph_replay(ctx):
+    """DECODE_GRAPH=1 replays the captured decode step (one graph per attention grid shape): the ids are those of
     the eager loop on every replay, across a change of grid shape, with eager work on other caches between the replays."""
     shape = Shape(dim=256, n_layers=2, n_heads=2, ffn_hidden=512, vocab_size=300, max_seq_len=460)
     W = synth_weights(shape, seed=61, std=0.08, norm_ones=False)
     gm = make_gpu(ctx, shape, W, True)
     prompt = np.random.default_rng(62).integers(0, shape.vocab_size, 376)
-    monkeypatch.delenv("RLLAMA_HIP_DECODE_GRAPH", raising=False)
     want, _, _ = gm.generate_greedy(prompt, 60, gm.make_caches())
-    monkeypatch.setenv("RLLAMA_HIP_DECODE_GRAPH", "1")
-    c = gm.make_caches()
-    got, _, _ = gm.generate_greedy(prompt, 20, c)           # positions 376 .. 395: the attention grid changes at 384
-    assert np.array_equal(got, want[:20])
-    for lo in (20, 40):
-        other = gm.make_caches()
-        gm.forward(prompt[:17], 0, other)                    # eager work between the replays (it drops the greedy state)
-        gm.forward([5], 17, other)
-        # token want[lo - 1] sits at position 376 + lo - 1; forwarding it again yields want[lo] and re-seeds the greedy state
-        assert gm.forward_greedy([int(want[lo - 1])], 376 + lo - 1, c) == want[lo]
-        if lo == 40:
-            c = c.true_clone()                               # a clone replays its own captures, not its source's
+    with options(ctx, DECODE_GRAPH="1"):
+        c = gm.make_caches()
+        got, _, _ = gm.generate_greedy(prompt, 20, c)           # positions 376 .. 395: the attention grid changes at 384
+        assert np.array_equal(got, want[:20])
+        for lo in (20, 40):
+            other = gm.make_caches()
+            gm.forward(prompt[:17], 0, other)                    # eager work between the replays (it drops the greedy state)
+            gm.forward([5], 17, other)
+            # token want[lo - 1] sits at position 376 + lo - 1; forwarding it again yields want[lo] and re-seeds the greedy state
             assert gm.forward_greedy([int(want[lo - 1])], 376 + lo - 1, c) == want[lo]
-        ids, _ = gm.decode_greedy(19, c)
-        assert np.array_equal(ids, want[lo + 1:lo + 20])
+            if lo == 40:
+                c = c.true_clone()                               # a clone replays its own captures, not its source's
+                assert gm.forward_greedy([int(want[lo - 1])], 376 + lo - 1, c) == want[lo]
+            ids, _ = gm.decode_greedy(19, c)
+            assert np.array_equal(ids, want[lo + 1:lo + 20])
     gm.free()
+
+
+@pytest.mark.parametrize("force_f16", [True, False], ids=["f16", "f32"])
+def test_decode_step_without_launches_for_the_embedding_row_and_the_pick(ctx, force_f16):
+    """A greedy decode step reads its embedding row inside layer 0's wq|wk|wv launch and makes its pick inside the output
+    head's launch (the last workgroup to finish reduces the workgroups' candidates and advances the token-step state).  With
+    DECODE_FOLD=0 both are launches of their own, as they were: same arithmetic on the same values, so the same ids, the same
+    logits bit for bit and the same cache rows -- eagerly and as a replayed graph, on a vocabulary that does not divide
+    into the workgroups evenly and one smaller than the grid."""
+    for vocab in (32003, 300):
+        shape = Shape(dim=256, n_layers=2, n_heads=2, ffn_hidden=512, vocab_size=vocab, max_seq_len=80)
+        W = synth_weights(shape, seed=63, std=0.08, norm_ones=False) if force_f16 else random_f32_weights(shape, 63)
+        gm = make_gpu(ctx, shape, W, force_f16)
+        prompt = np.random.default_rng(64).integers(0, vocab, 9)
+        runs = {}
+        for name, opts in (("separate", dict(DECODE_FOLD="0")), ("folded", {}), ("folded-graph", dict(DECODE_GRAPH="1"))):
+            with options(ctx, **opts):
+                c = gm.make_caches()
+                ids, _, _ = gm.generate_greedy(prompt, 40, c)
+                more, _ = gm.decode_greedy(20, c)
+                last = gm.forward([int(more[-1])], 9 + 40 + 20 - 1, c)   # the logits behind the next pick
+                runs[name] = (np.concatenate([ids, more]), last, c.read(1, 1, 0), c.read(1, 1, 1))
+        for name in ("folded", "folded-graph"):
+            assert np.array_equal(runs[name][0], runs["separate"][0]), (vocab, name)
+            for a, b in zip(runs[name][1:], runs["separate"][1:]):
+                assert np.array_equal(a, b), (vocab, name)
+        gm.free()
 
 
 @pytest.mark.parametrize("n_prompt", [200, 1100], ids=["200-tokens", "1100-tokens"])

@@ -497,3 +497,100 @@ def test_golden_tiny_reproduced():
         toks = fx[mode]["tokens"]
         assert np.allclose(om.forward(toks[:7], 0, oc), _bits_to_f32(fx[mode]["logits_after_7_f32_bits"]), rtol=1e-6, atol=1e-7)
         assert np.allclose(om.forward(toks[7:8], 7, oc), _bits_to_f32(fx[mode]["logits_after_8_f32_bits"]), rtol=1e-6, atol=1e-7)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# The exact-sum probe (oracle.set_exact_sums): what the reference's arithmetic gives when no fp32 addition inside a sum
+# rounds.  It is the yardstick of the full-depth GPU tests, so it is pinned here like the oracle proper.
+# ---------------------------------------------------------------------------------------------------------
+@pytest.fixture
+def exact_sums():
+    oracle.set_exact_sums(True)
+    try:
+        yield
+    finally:
+        oracle.set_exact_sums(False)
+
+
+def test_exact_sums_are_the_correctly_rounded_sums(exact_sums):
+    """Dot products against math.fsum of the exact products (products of two f32 are exact in float64), rounded to f32 once:
+    a dropped term, a product rounded to f32 first, or an fp32 accumulator each fail on these vectors."""
+    import math
+    rng = np.random.default_rng(41)
+    for k in (1, 7, 8, 9, 64, 333, 4096, 11008):
+        a = (rng.standard_normal(k) * 3).astype(np.float32)
+        b = rng.standard_normal(k).astype(np.float32)
+        want = np.float32(math.fsum(float(x) * float(y) for x, y in zip(a, b)))
+        assert np.float32(oracle.dot8_f32(a, b)) == want, k
+        ah, bh = a.astype(np.float16), b.astype(np.float16)
+        want_h = np.float32(math.fsum(float(x) * float(y) for x, y in zip(ah, bh)))
+        assert np.float32(oracle.dot8_f16(ah.view(np.uint16), bh.view(np.uint16))) == want_h, k
+    # a sum where every fp32 accumulation order loses the small terms and float64 keeps them
+    a = np.array([1.0] + [2.0 ** -25] * 64, np.float32)
+    b = np.ones(65, np.float32)
+    assert oracle.dot8_f32(a, b) == float(np.float32(1.0 + 64 * 2.0 ** -25))
+    oracle.set_exact_sums(False)
+    assert oracle.dot8_f32(a, b) != float(np.float32(1.0 + 64 * 2.0 ** -25))
+    oracle.set_exact_sums(True)
+    # the matrix forms go through the same sums
+    x = rng.standard_normal((3, 100)).astype(np.float32)
+    w = rng.standard_normal((5, 100)).astype(np.float32)
+    want = np.array([[np.float32(math.fsum(float(p) * float(q) for p, q in zip(xr, wr))) for wr in w] for xr in x], np.float32)
+    assert np.array_equal(oracle.matmul_transposed_f32(x, w), want)
+    xh, wh = x.astype(np.float16), w.astype(np.float16)
+    want_h = np.array([[np.float32(math.fsum(float(p) * float(q) for p, q in zip(xr, wr))) for wr in wh] for xr in xh], np.float32)
+    got_h = oracle.matmul_transposed_f16(xh.view(np.uint16), wh.view(np.uint16)).view(np.float16)
+    assert np.array_equal(got_h, want_h.astype(np.float16))           # f32 first, then f16: the reference's two roundings
+    kq = rng.standard_normal(24).astype(np.float32)
+    km = rng.standard_normal((24, 13)).astype(np.float32)
+    want_v = np.array([np.float32(math.fsum(float(kq[r]) * float(km[r, c]) for r in range(24))) for c in range(13)], np.float32)
+    assert np.array_equal(oracle.vector_matrix_mul_f32(kq, km), want_v)
+    assert np.array_equal(oracle.matmul_f32_seqk(kq.reshape(1, -1), km)[0], want_v)
+
+
+def test_exact_sums_leave_everything_but_the_sums_alone(exact_sums):
+    """RMSNorm and softmax keep the reference's f32 element-wise steps and libm calls; only the sum changes."""
+    import math
+    rng = np.random.default_rng(42)
+    x = (rng.standard_normal(1000) * 2).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 1000).astype(np.float32)
+    ss = np.float32(math.fsum(float(v) * float(v) for v in x))
+    rs = np.float32(1.0) / np.sqrt(np.float32(ss / np.float32(1000) + np.float32(1e-6)))
+    want = (x * rs) * w                                               # two f32 roundings per element (tensor.rs:631, 672)
+    assert np.array_equal(oracle.rmsnorm_row(x, w, 1e-6), want)
+    s = rng.standard_normal(300).astype(np.float32)
+    oracle.set_exact_sums(False)
+    plain = oracle.softmax_row(s)
+    oracle.set_exact_sums(True)
+    got = oracle.softmax_row(s)
+    # every ratio got / plain is one constant (the two denominators), to within the rounding of the divisions
+    ratio = got.astype(np.float64) / plain.astype(np.float64)
+    assert np.ptp(ratio) < 3e-7
+    assert abs(float(np.sum(got.astype(np.float64))) - 1.0) < 2e-7    # the float64 denominator normalises better than 300 fp32 adds would need to
+
+
+@pytest.mark.parametrize("shape", [TINY, SMALL], ids=["tiny", "small"])
+def test_exact_sum_forward_sits_between_the_oracle_and_float64(shape, exact_sums):
+    """Whole forward, f16 mode: with exact sums the restatement must land (much) closer to the independent float64 model with
+    the same rounding points than the reference's own fp32 lane order does; f32 mode: closer still."""
+    W = synth_weights(shape, seed=3, std=0.08, norm_ones=False)
+    rng = np.random.default_rng(13)
+    toks = rng.integers(0, shape.vocab_size, 8)
+    for force_f16 in (False, True):
+        m = make_oracle(shape, W, force_f16)
+        ref = RefF64(shape, W, f16_points=force_f16, via_f32=True)
+        c = m.make_caches()
+        got = [m.forward(toks[:5], 0, c)] + [m.forward(toks[i:i + 1], i, c) for i in range(5, 8)]
+        want = [ref.forward(toks[:5], 0)] + [ref.forward(toks[i:i + 1], i) for i in range(5, 8)]
+        oracle.set_exact_sums(False)
+        try:
+            c2 = m.make_caches()
+            plain = [m.forward(toks[:5], 0, c2)] + [m.forward(toks[i:i + 1], i, c2) for i in range(5, 8)]
+        finally:
+            oracle.set_exact_sums(True)
+        d_exact = max(max_rel_err(a, b) for a, b in zip(got, want))
+        d_plain = max(max_rel_err(a, b) for a, b in zip(plain, want))
+        if force_f16:
+            assert d_exact < 0.25 * d_plain < 1e-2, (d_exact, d_plain)   # measured: 1.7e-7 / 2.0e-5 against 4.6e-4 / 8.2e-4
+        else:
+            assert d_exact < 2e-6 and d_exact < d_plain, (d_exact, d_plain)
