@@ -76,7 +76,7 @@ HOST_BIN = os.path.join(HERE, "host", "rllama_generate")
 def build_host(force: bool = False) -> str:
     """Compiles the C++ host example (header-only mirror of the reference API + the token loop) against the library."""
     src = os.path.join(HERE, "host", "generate_main.cpp")
-    hdrs = [os.path.join(HERE, "host", "rllama_hip.hpp"), os.path.join(HERE, "host", "model_files.hpp"), os.path.join(HERE, "host", "tokenizer.hpp")]
+    hdrs = [os.path.join(HERE, "host", h) for h in ("rllama_hip.hpp", "model_files.hpp", "tokenizer.hpp", "file_tools.hpp")]
     if not force and os.path.exists(HOST_BIN) and all(os.path.getmtime(HOST_BIN) >= os.path.getmtime(f) for f in (src, *hdrs, LIB)):
         return HOST_BIN
     cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-Wextra", src, "-o", HOST_BIN, "-L" + HERE, "-lrllama_hip", "-Wl,-rpath,$ORIGIN/.."]
@@ -86,6 +86,27 @@ def build_host(force: bool = False) -> str:
     return HOST_BIN
 
 
+ASAN_BIN = os.path.join(HERE, "host", "rllama_check_files_asan")
+ASAN_FLAGS = ["-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-static-libasan", "-static-libubsan"]
+
+
+def build_host_asan(force: bool = False) -> str:
+    """The host-only file readers (pickle subset, params.json, shard joining, tokenizer model file) as a program built with
+    AddressSanitizer and UndefinedBehaviorSanitizer.  CPU code only: nothing of the device library is in it."""
+    src = os.path.join(HERE, "host", "check_files_main.cpp")
+    hdrs = [os.path.join(HERE, "host", h) for h in ("rllama_hip.hpp", "model_files.hpp", "tokenizer.hpp", "file_tools.hpp")]
+    if not force and os.path.exists(ASAN_BIN) and all(os.path.getmtime(ASAN_BIN) >= os.path.getmtime(f) for f in (src, *hdrs)):
+        return ASAN_BIN
+    cmd = ["g++", *ASAN_FLAGS, "-std=c++17", "-Wall", "-Wextra", src, "-o", ASAN_BIN]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("sanitizer build of the host readers failed:\n" + " ".join(cmd) + "\n" + r.stdout + r.stderr)
+    return ASAN_BIN
+
+
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv))
-    print(build_host(force="--force" in sys.argv))
+    if "--host-asan" in sys.argv:
+        print(build_host_asan(force=True))
+    else:
+        print(build(force="--force" in sys.argv))
+        print(build_host(force="--force" in sys.argv))

@@ -14,6 +14,7 @@
 //
 // It exists to show (and to compile-check in every build) that the header-only host layer needs nothing but
 // the C ABI.  Exits non-zero with the library's message if there is no gfx950 device.
+#include "file_tools.hpp"
 #include "model_files.hpp"
 #include "rllama_hip.hpp"
 #include "tokenizer.hpp"
@@ -22,52 +23,9 @@
 #include <cstdlib>
 #include <random>
 
-static int inspect(const char *dir) {
-    using namespace rllama;
-    const DataSource src = DataSource::from_inferred_source(dir);
-    const ModelParams mp = src.params();
-    printf("params dim=%zu n_heads=%zu n_layers=%zu norm_eps=%g vocab_size=%lld shards=%zu\n", mp.dim, mp.n_heads, mp.n_layers, mp.norm_eps,
-           (long long)mp.vocab_size, src.unpickled().size());
-    if (src.unpickled().empty()) return 0;
-    for (const auto &kv : src.unpickled()[0]->entries) {
-        const std::string &name = kv.first;
-        // how the reference joins the shards of this tensor (src/transformer.rs:490-503, 595-614; src/embedding.rs:37)
-        const bool cols = name.find(".wo.") != std::string::npos || name.find(".w2.") != std::string::npos || name == "tok_embeddings.weight";
-        const bool first = name.find("norm") != std::string::npos;
-        const HalfMatrix m = load_from_pieces(src, name, cols ? FromPiecesDirection::Cols : FromPiecesDirection::Rows, first);
-        uint64_t h = 1469598103934665603ull; // FNV-1a over the little-endian bytes
-        for (uint16_t b : m.bits) {
-            h = (h ^ (b & 0xff)) * 1099511628211ull;
-            h = (h ^ (b >> 8)) * 1099511628211ull;
-        }
-        printf("tensor %s %lld %lld %016llx\n", name.c_str(), (long long)m.rows, (long long)m.cols, (unsigned long long)h);
-    }
-    return 0;
-}
-
 int main(int argc, char **argv) {
-    if (argc >= 3 && std::string(argv[1]) == "--inspect") {
-        try {
-            return inspect(argv[2]);
-        } catch (const std::exception &e) {
-            fprintf(stderr, "rllama_generate: %s\n", e.what());
-            return 1;
-        }
-    }
-    if (argc >= 4 && std::string(argv[1]) == "--tokenize") {
-        try {
-            const rllama::Tokenizer tok = rllama::Tokenizer::load(argv[2]);
-            printf("ids:");
-            for (rllama::TokenId t : tok.tokenize_to_ids(argv[3])) printf(" %d", t);
-            printf("\n");
-            for (rllama::TokenId t : tok.tokenize_to_ids(argv[3]))
-                if (t != 1) printf("piece %d %s\n", t, tok.id_to_str(t).c_str());
-            return 0;
-        } catch (const std::exception &e) {
-            fprintf(stderr, "rllama_generate: %s\n", e.what());
-            return 1;
-        }
-    }
+    if (argc >= 3 && std::string(argv[1]) == "--inspect") return rllama::tools::guarded("rllama_generate", [&] { return rllama::tools::inspect(argv[2]); });
+    if (argc >= 4 && std::string(argv[1]) == "--tokenize") return rllama::tools::guarded("rllama_generate", [&] { return rllama::tools::tokenize(argv[2], argv[3]); });
     bool use_sampler = false;
     rllama::TokenSampler sampler;
     if (argc >= 6 && std::string(argv[1]) == "--sample") {

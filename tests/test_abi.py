@@ -58,6 +58,80 @@ def test_rust_ffi_crate_matches_the_header():
                                          "rlh_tensor_kind", "rlh_status", "rlh_dtype"), f"the integration guide names {name}, which the header does not declare"
 
 
+def _ctypes_of_rust(t: str):
+    """The ctypes type a Rust FFI type corresponds to (what the C ABI passes for it)."""
+    import ctypes as C
+    scalars = {"c_int": C.c_int, "c_float": C.c_float, "c_double": C.c_double, "i32": C.c_int32, "u16": C.c_uint16, "u64": C.c_uint64, "usize": C.c_size_t,
+               "f32": C.c_float, "f64": C.c_double}
+    t = t.strip()
+    if t in scalars:
+        return scalars[t]
+    m = re.match(r"^\*(const|mut) (.*)$", t)
+    assert m, t
+    inner = m.group(2).strip()
+    if inner == "c_char":
+        return C.c_char_p
+    if inner == "c_void" or inner in ("rlh_ctx", "rlh_model", "rlh_caches", "rlh_tensor", "rlh_event"):
+        return C.c_void_p                                   # opaque handles and untyped buffers
+    if inner == "rlh_model_params":
+        return C.POINTER(_lib.ModelParams)
+    if inner == "rlh_sampler_params":
+        return C.POINTER(_lib.SamplerParams)
+    return C.POINTER(_ctypes_of_rust(inner))
+
+
+def test_rust_ffi_types_match_the_ctypes_tables():
+    """Neither cargo nor rustc exists where this suite runs, so the generated crate is never compiled here.  What can be
+    checked without a compiler: every argument and return type of every function, and every field (type and order) of the two
+    #[repr(C)] structs, denote the same C type as the ctypes tables that the whole GPU suite calls through; and the struct
+    layouts ctypes computes are the C compiler's (sizes and offsets of include/rllama_hip.h compiled with gcc)."""
+    import ctypes as C
+    import subprocess
+    import tempfile
+    root = os.path.dirname(HERE)
+    lib_rs = open(os.path.join(root, "rust", "rllama-hip-sys", "src", "lib.rs")).read()
+    decls = {m.group(1): (m.group(2), m.group(3)) for m in re.finditer(r"pub fn (rlh_[a-z0-9_]+)\((.*?)\)(?: -> ([^;]+))?;", lib_rs)}
+    assert sorted(decls) == sorted(_lib.SIGNATURES)
+    same = lambda a, b: a is b or (C.sizeof(a) == C.sizeof(b) and a._type_ == b._type_ and not hasattr(a, "contents") and not hasattr(b, "contents"))  # c_int is c_int32 here
+    for name, (res, args) in _lib.SIGNATURES.items():
+        params, ret = decls[name]
+        rust_args = [a.split(":", 1)[1] for a in params.split(",")] if params.strip() else []
+        assert len(rust_args) == len(args), name
+        for i, (ra, ca) in enumerate(zip(rust_args, args)):
+            got = _ctypes_of_rust(ra)
+            ok = got is ca or (hasattr(got, "_type_") and hasattr(ca, "_type_") and getattr(got, "_type_", None) == getattr(ca, "_type_", None)) or \
+                (hasattr(got, "contents") and hasattr(ca, "contents") and C.sizeof(got._type_) == C.sizeof(ca._type_) and getattr(got._type_, "_type_", 0) == getattr(ca._type_, "_type_", 1))
+            assert ok, f"{name} argument {i}: Rust `{ra.strip()}` is {got}, the ctypes table has {ca}"
+        want_ret = None if ret is None else _ctypes_of_rust(ret)
+        assert (want_ret is None and res is None) or want_ret is res or same(want_ret, res), (name, ret, res)
+    for sname, table in (("rlh_model_params", _lib.ModelParams), ("rlh_sampler_params", _lib.SamplerParams)):
+        body = re.search(r"pub struct %s \{(.*?)\}" % sname, lib_rs, flags=re.S).group(1)
+        fields = [(m.group(1), m.group(2)) for m in re.finditer(r"pub ([a-z_0-9]+): ([^,]+),", body)]
+        assert [f for f, _ in fields] == [f for f, _ in table._fields_], sname          # same fields in the same order
+        for (fname, rtype), (_, ctype) in zip(fields, table._fields_):
+            got = _ctypes_of_rust(rtype)
+            assert got is ctype or same(got, ctype), (sname, fname, rtype, ctype)
+    # ctypes' layout of the two structs against gcc's of the header itself
+    prog = '''#include <stdio.h>
+#include <stddef.h>
+#include "rllama_hip.h"
+int main(void) {
+    printf("%zu %zu %zu %zu %zu\\n", sizeof(rlh_model_params), offsetof(rlh_model_params, norm_eps), offsetof(rlh_model_params, force_f16),
+           offsetof(rlh_model_params, percentage_to_gpu), offsetof(rlh_model_params, max_seq_len));
+    printf("%zu %zu %zu\\n", sizeof(rlh_sampler_params), offsetof(rlh_sampler_params, top_k), offsetof(rlh_sampler_params, repetition_penalty));
+    return 0;
+}
+'''
+    with tempfile.TemporaryDirectory() as d:
+        src, exe = os.path.join(d, "layout.c"), os.path.join(d, "layout")
+        open(src, "w").write(prog)
+        subprocess.check_call(["gcc", "-I", os.path.join(root, "include"), src, "-o", exe])
+        out = subprocess.check_output([exe], text=True).split()
+    M, S = _lib.ModelParams, _lib.SamplerParams
+    assert [int(v) for v in out] == [C.sizeof(M), M.norm_eps.offset, M.force_f16.offset, M.percentage_to_gpu.offset, M.max_seq_len.offset,
+                                     C.sizeof(S), S.top_k.offset, S.repetition_penalty.offset]
+
+
 def test_no_oracle_in_product():
     """The shipped package and library must not reach into oracle/ (test infrastructure)."""
     pkg = os.path.dirname(_lib.__file__)

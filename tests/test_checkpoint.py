@@ -59,12 +59,15 @@ def test_unpickle_opcode_details():
     assert ck.unpickle(b"\x80\x02K\x07") == 7
 
 
-@pytest.mark.parametrize("data,msg", [
+REJECTED_PICKLES = [
     (b"", "too short"), (b"\x80\x03K\x01.", "magic"), (b"\x80\x02\x8a\x01\x01.", "Unknown opcode: 138"), (b"\x80\x02K\x01K\x02\x87.", "Unknown opcode: 135"),
     (b"\x80\x02K\x01K\x02.", "exactly one"), (b"\x80\x02K\x01t.", "No mark"), (b"\x80\x02h\x00.", "BINGET index"), (b"\x80\x02X\x05\x00\x00\x00ab", "BINUNICODE"),
     (b"\x80\x02K\x01(K\x02K\x03u.", "SETITEMS on non-dict"), (b"\x80\x02}(K\x01u.", "Unexpected mark"), (b"\x80\x02J\x01\x02", "BININT"),
     (b"\x80\x02N.", "Unknown opcode: 78"),
-])
+]
+
+
+@pytest.mark.parametrize("data,msg", REJECTED_PICKLES)
 def test_unpickle_rejects(data, msg):
     with pytest.raises(ck.UnpicklingError, match=msg):
         ck.unpickle(data)
@@ -272,7 +275,7 @@ def _hostile_dir(tmp_path, tag, entries_by_shard, files):
     return str(path)
 
 
-@pytest.mark.parametrize("tag,entries,msg", [
+DAMAGED_CHECKPOINTS = [
     # negative extents (BININT is signed, src/unpickler.rs:414): one shard claims 6 columns, the other -4, so the sum (2) would
     # size the joined matrix while the first shard still copies 6 columns per row
     ("mixed_sign_cols", [[("w", "0", (3, 6))], [("w", "0", (3, -4))]], "invalid stride|does not fit its storage"),
@@ -284,7 +287,10 @@ def _hostile_dir(tmp_path, tag, entries_by_shard, files):
     # the storage key must stay a file name inside consolidated.NN/data/
     ("dotdot_key", [[("w", "../../params.json", (1, 2))]], "not a plain file name"),
     ("absolute_key", [[("w", "/etc/hostname", (1, 2))]], "not a plain file name"),
-])
+]
+
+
+@pytest.mark.parametrize("tag,entries,msg", DAMAGED_CHECKPOINTS)
 def test_damaged_checkpoints_fail_cleanly_in_both_readers(tmp_path, tag, entries, msg):
     """Extents and storage keys come from the pickle unchecked; both readers must refuse them before sizing a buffer or
     opening a path (the reference panics on the same inputs: usize casts of negative i64 and slice bounds)."""

@@ -14,9 +14,10 @@ and three distances are reported: device <-> oracle (what the task's tolerance i
 reference itself sits from its own exact-sum result: f16 rounding decisions flipped by fp32 summation noise, compounding
 through the residual stream) and device <-> exact.  Bars: device <-> oracle within 1e-2 of the largest |logit| (1e-4 in f32
 mode) at every call -- at the 80 layers of the 65B shape within 1.5e-2, see that test; device <-> exact no larger than
-1.25 x oracle <-> exact; the residual stream after every layer no further from the exact one than 1.5 x the oracle's is
-(+ a floor) and without a jump from one layer to the next; every block alone, fed the oracle's own input stream, within 2e-3
-of the oracle's output stream; greedy ids identical wherever the oracle's own top-2 gap is larger than twice the measured
+1.25 x oracle <-> exact (2 x in f32 mode, where both sit below a fifth of the tolerance); the residual stream after every
+layer no further from the exact one than 1.5 x (f32 mode: 2 x) the oracle's is (+ a floor) and without a jump from one layer
+to the next; every block alone, fed the oracle's own input stream, within 2e-3 (f32 mode: 1e-5) of the oracle's output
+stream; greedy ids identical wherever the oracle's own top-2 gap is larger than twice the measured
 difference, and where the two loops part at a step without such a gap, the device's pick is one of the oracle's top two.
 """
 import json
@@ -157,13 +158,13 @@ def run_full_depth(ctx, name, dim, n_layers, n_heads, ffn, vocab, n_prompt, n_de
         assert max(d_de) <= exact_factor * max(d_oe) + floor, \
             f"{name}: the device is {max(d_de):.3e} from the exact-sum result, the reference's own arithmetic {max(d_oe):.3e}"
     if with_taps:
-        per_block = 2e-3 if force_f16 else 2e-6
+        per_block = 2e-3 if force_f16 else 1e-5   # (fp32 sums of 4096 to 11008 terms in two orders: a few 1e-6 at the 7B dimensions)
         assert max(block_err) < per_block, f"{name}: block {int(np.argmax(block_err))} alone is {max(block_err):.3e} from the oracle's output stream"
         for l in range(1, n_layers):   # no jump from one layer to the next (a wrong tile or split shows as one)
             assert t_do[l] < 2.5 * t_do[l - 1] + (1e-3 if force_f16 else 1e-6), (name, l, t_do[l - 1], t_do[l])
         if with_exact:
             for l in range(n_layers):
-                assert t_de[l] <= 1.5 * t_oe[l] + (5e-4 if force_f16 else 5e-7), (name, l, t_de[l], t_oe[l])
+                assert t_de[l] <= (1.5 if force_f16 else 2.0) * t_oe[l] + (5e-4 if force_f16 else 1e-6), (name, l, t_de[l], t_oe[l])
     assert g_ids[:first_unclear] == o_ids[:first_unclear], (g_ids, o_ids, gaps, abs_diff)
     if g_ids != o_ids:
         # the loops part at a step whose top-2 gap is within the measured difference: the device's pick there must be
@@ -193,7 +194,7 @@ def test_full_depth_7b_f32_mode_against_the_oracle(ctx):
     free_gb = os.sysconf("SC_AVPHYS_PAGES") * os.sysconf("SC_PAGE_SIZE") / 1e9
     if free_gb < 70:
         pytest.skip(f"host has {free_gb:.0f} GB free; the oracle's fp32 copy of the 7B weights needs 27 GB, and as much while it is handed over")
-    run_full_depth(ctx, "c1_7b_f32", 4096, 32, 32, 11008, 32000, 8, 8, force_f16=False)
+    run_full_depth(ctx, "c1_7b_f32", 4096, 32, 32, 11008, 32000, 8, 8, force_f16=False, exact_factor=2.0)
 
 
 @pytest.mark.timeout(600)

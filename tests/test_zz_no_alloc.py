@@ -48,3 +48,32 @@ def test_attn_decode_noalloc_rejects_sizes_beyond_its_work_memory(ctx):
     q.attn_decode_noalloc(out, z, z, H, S, 128, n_splits=63)      # 1,048,320 floats fit
     with pytest.raises(rllama_amd.RllamaHipError):
         q.attn_decode_noalloc(out, z, z, H, S, S + 1)             # the checks of rlh_attn_decode apply
+
+
+def test_attn_decode_noalloc_allocates_nothing(ctx):
+    """What the entry point exists for: no device allocation inside the call.  The free device memory the HIP runtime reports
+    (hipMemGetInfo, called on the runtime library this process already has loaded) does not move over 50 calls at growing
+    split counts, where the allocating entry point, asked for more work memory than it holds, makes it move."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+
+    def free_bytes():
+        ctx.sync()
+        free, total = C.c_size_t(0), C.c_size_t(0)
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    rng = np.random.default_rng(43)
+    H, hd, S, T = 64, 128, 2048, 2040
+    q, ck, cv = _case(ctx, rng, H, hd, S, True)
+    out = Tensor.zeros(ctx, 1, H * hd, TensorDType.Float32)
+    q.attn_decode_noalloc(out, ck, cv, H, S, T, n_splits=2)       # first use
+    before = free_bytes()
+    for i in range(50):
+        q.attn_decode_noalloc(out, ck, cv, H, S, T, n_splits=2 + i % 62)
+    assert free_bytes() == before
+    # the probe does see an allocation of the size in question: 64 heads x 64 splits x 130 floats = 2.1 MB of work memory
+    held = Tensor.zeros(ctx, 64 * 64, 130 * 4, TensorDType.Float32)      # 8.5 MB: more than the allocator's granularity
+    assert free_bytes() < before
+    held.free()
