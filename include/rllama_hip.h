@@ -312,6 +312,16 @@ int  rlh_model_time_kernel(rlh_model *model, rlh_caches *caches, int which, int 
 int  rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int round_x, int round_y, int n_buffers, int iters,
                    float *us_per_launch);
 
+/* Where the fixed cost of a GEMV launch is spent: `launches` back-to-back launches of the isolated product (as rlh_time_gemv,
+ * f16 weights, n_buffers distinct matrices) in which every wavefront reads the 100 MHz wall clock at kernel entry, when the
+ * activation vector is staged, behind its first and its last burst of weights, and at exit.  out_us receives 8 means over
+ * the launches after the first, in microseconds: [0] first wavefront of a launch enters after the last wavefront of the
+ * previous launch left (the gap between dependent kernels on the device), [1] last wavefront enters after the first one
+ * (dispatch ramp), [2] entry -> x staged (prologue, mean over wavefronts), [3] x staged -> first burst consumed (first-byte
+ * latency, mean), [4] first -> last burst consumed (streaming, mean), [5] last burst -> exit (epilogue, mean), [6] first
+ * wavefront to leave -> last wavefront to leave (tail skew), [7] first entry -> last exit (the launch as the device sees it). */
+int  rlh_probe_gemv_phases(rlh_ctx *ctx, int rows, int k, int n_buffers, int launches, float *out_us);
+
 /* ------------------------------------------------------------------------------------------------
  * Synthetic inputs (host side; usable without a device).  See synth.h.
  * ---------------------------------------------------------------------------------------------- */

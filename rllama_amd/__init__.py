@@ -73,6 +73,14 @@ class Context:
         check(self._lib.rlh_time_gemv(self._h, rows, k, dtype, 1 if round_x else 0, 1 if round_y else 0, n_buffers, iters, C.byref(us)))
         return us.value
 
+    GEMV_PHASES = ("gap_after_previous_launch", "dispatch_ramp", "prologue", "first_byte_latency", "streaming", "epilogue", "tail_skew", "first_entry_to_last_exit")
+
+    def probe_gemv_phases(self, rows: int, k: int, n_buffers: int = 12, launches: int = 64):
+        """Microseconds of each phase of the isolated f16 GEMV launch, from wall-clock readings inside the kernel."""
+        out = (C.c_float * 8)()
+        check(self._lib.rlh_probe_gemv_phases(self._h, rows, k, n_buffers, launches, out))
+        return dict(zip(self.GEMV_PHASES, (round(float(v), 3) for v in out)))
+
     def close(self) -> None:
         """Ends the context.  Handles made from it are dead afterwards (their free() becomes a no-op)."""
         if getattr(self, "_h", None):

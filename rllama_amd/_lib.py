@@ -97,6 +97,7 @@ SIGNATURES = {
     "rlh_argmax_greedy": (C.c_int, [_vp, C.c_float, _i32p]),
     "rlh_model_time_kernel": (C.c_int, [_vp, _vp, C.c_int, C.c_int, C.c_int, _fp, C.POINTER(C.c_uint64)]),
     "rlh_time_gemv": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _fp]),
+    "rlh_probe_gemv_phases": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.c_int, _fp]),
     "rlh_synth_normal_f16": (None, [C.c_uint64, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_double, C.POINTER(C.c_uint16)]),
     "rlh_synth_tokens": (None, [C.c_uint64, C.c_uint64, C.c_uint64, C.c_int32, C.c_int32, _i32p]),
     "rlh_abi_version": (C.c_int, []),

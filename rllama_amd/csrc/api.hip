@@ -10,6 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdarg>
@@ -1642,6 +1643,87 @@ extern "C" int rlh_time_gemv(rlh_ctx *ctx, int rows, int k, int w_dtype, int rou
     HIP_TRY(e);
     HIP_TRY(e2);
     *us_per_launch = ms * 1000.0f / (float)iters;
+    return RLH_OK;
+}
+
+extern "C" int rlh_probe_gemv_phases(rlh_ctx *ctx, int rows, int k, int n_buffers, int launches, float *out_us) {
+    if (!ctx || !out_us || rows < 1 || k < 8 || k % 8 != 0 || n_buffers < 1 || launches < 2 || launches > 256) return fail(RLH_ERR_INVALID, "rlh_probe_gemv_phases: bad argument");
+    CtxLock lock(ctx);
+    hipStream_t st = ctx->stream;
+    const size_t wbytes = (size_t)rows * k * 2;
+    std::vector<void *> bufs((size_t)n_buffers, nullptr);
+    float *x = nullptr, *y = nullptr;
+    unsigned long long *stamps = nullptr;
+    constexpr int kS = 5;
+    const size_t max_waves = 2048 + 64;
+    hipError_t e = hipSuccess;
+    for (int i = 0; e == hipSuccess && i < n_buffers; i++) {
+        e = hipMalloc(&bufs[(size_t)i], wbytes);
+        if (e == hipSuccess) e = launch_synth_fill(bufs[(size_t)i], 1, (uint64_t)rows * k, synth_key(98, (uint64_t)i), 0.02, st);
+    }
+    if (e == hipSuccess) e = hipMalloc((void **)&x, sizeof(float) * (size_t)k);
+    if (e == hipSuccess) e = hipMalloc((void **)&y, sizeof(float) * (size_t)rows);
+    if (e == hipSuccess) e = hipMalloc((void **)&stamps, sizeof(unsigned long long) * (size_t)launches * max_waves * kS);
+    if (e == hipSuccess) e = hipMemsetAsync(stamps, 0, sizeof(unsigned long long) * (size_t)launches * max_waves * kS, st);
+    if (e == hipSuccess) e = launch_fill_f32(x, (uint64_t)k, 0.5f, st);
+    GemvParams p{};
+    p.w_is_f16 = 1;
+    p.x = x;
+    p.y = y;
+    p.n_rows = rows;
+    p.k = k;
+    p.stream_weights = 1;
+    int n_waves = 0;
+    for (int i = 0; e == hipSuccess && i < launches; i++) {
+        p.w = bufs[(size_t)(i % n_buffers)];
+        p.stamps = stamps + (size_t)i * max_waves * kS;
+        e = launch_gemv_stamped(p, st, &n_waves);
+    }
+    std::vector<unsigned long long> host;
+    if (e == hipSuccess && (size_t)n_waves > max_waves) e = hipErrorInvalidValue;
+    if (e == hipSuccess) {
+        host.resize((size_t)launches * max_waves * kS);
+        e = hipMemcpyAsync(host.data(), stamps, host.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost, st);
+    }
+    hipError_t e2 = hipStreamSynchronize(st);
+    for (void *b : bufs)
+        if (b) (void)hipFree(b);
+    for (void *b : {(void *)x, (void *)y, (void *)stamps})
+        if (b) (void)hipFree(b);
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    unsigned long long prev_last_exit = 0;
+    int counted = 0;
+    for (int i = 0; i < launches; i++) {
+        const unsigned long long *s = host.data() + (size_t)i * max_waves * kS;
+        unsigned long long first_in = ~0ull, last_in = 0, first_out = ~0ull, last_out = 0;
+        double pro = 0, lat = 0, stream = 0, epi = 0;
+        for (int w = 0; w < n_waves; w++) {
+            const unsigned long long *t = s + (size_t)w * kS;
+            first_in = std::min(first_in, t[0]);
+            last_in = std::max(last_in, t[0]);
+            first_out = std::min(first_out, t[4]);
+            last_out = std::max(last_out, t[4]);
+            pro += (double)(t[1] - t[0]);
+            lat += (double)(t[2] - t[1]);
+            stream += (double)(t[3] - t[2]);
+            epi += (double)(t[4] - t[3]);
+        }
+        if (i > 0) {
+            acc[0] += (double)first_in - (double)prev_last_exit;
+            acc[1] += (double)(last_in - first_in);
+            acc[2] += pro / n_waves;
+            acc[3] += lat / n_waves;
+            acc[4] += stream / n_waves;
+            acc[5] += epi / n_waves;
+            acc[6] += (double)(last_out - first_out);
+            acc[7] += (double)(last_out - first_in);
+            counted++;
+        }
+        prev_last_exit = last_out;
+    }
+    for (int j = 0; j < 8; j++) out_us[j] = (float)(acc[j] / counted * 0.01); // 100 MHz ticks -> microseconds
     return RLH_OK;
 }
 

@@ -31,7 +31,7 @@ size_t gemv_lds_bytes(int k, int w_is_f16, int x_f16) {
     return (size_t)gemv_iters(k, vec) * kWave * vec * (x_f16 ? 2 : 4);
 }
 
-template <typename WT, typename XT, int kEpi, bool kStream, int kBurst = kGemvBurst>
+template <typename WT, typename XT, int kEpi, bool kStream, int kBurst = kGemvBurst, bool kEmbed = false, bool kStamp = false>
 __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     extern __shared__ uint4_t smem_raw[];
     __shared__ float red[16];
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     // (measured: issuing the first burst behind the prologue's loads is worth 1 % on the w1|w3 product, nothing or a loss on
     // the others, so only that instantiation does it)
     constexpr int kPre = (RLH_GEMV_PRELOAD && kEpi == kEpiSilu) ? kPreSelf : kPreNone;
-    gemv_body<WT, XT, kEpi, kStream, kPre, kBurst>(p, smem_raw, red, rope_f);
+    gemv_body<WT, XT, kEpi, kStream, kPre, kBurst, kEmbed, kStamp>(p, smem_raw, red, rope_f);
 }
 
 static int gemv_blocks(int n_units) {
@@ -83,6 +83,14 @@ static hipError_t launch_gemv_t(GemvParams p, hipStream_t s) {
             if (pieces % 7 == 0) return pick(std::integral_constant<int, 7>{});
         }
     }
+    if constexpr (kEpi == kEpiRopeKv) {
+        // layer 0 of a token step: the input row read from the embedding table (an instantiation of its own, so that the other
+        // layers' kernel carries none of it)
+        if (p.embed_table != nullptr) {
+            if (p.stream_weights) return launch(gemv_kernel<WT, XT, kEpi, true, kGemvBurst, true>);
+            return launch(gemv_kernel<WT, XT, kEpi, false, kGemvBurst, true>);
+        }
+    }
     if (p.stream_weights) return launch(gemv_kernel<WT, XT, kEpi, true>);
     return launch(gemv_kernel<WT, XT, kEpi, false>);
 }
@@ -93,6 +101,20 @@ static hipError_t launch_gemv_e(const GemvParams &p, hipStream_t s) {
         return p.x_f16 ? launch_gemv_t<half_t, half_t, kEpi>(p, s) : launch_gemv_t<half_t, float, kEpi>(p, s);
     }
     return p.x_f16 ? launch_gemv_t<float, half_t, kEpi>(p, s) : launch_gemv_t<float, float, kEpi>(p, s);
+}
+
+hipError_t launch_gemv_stamped(const GemvParams &p, hipStream_t s, int *n_waves) {
+    if (!p.w_is_f16 || p.x_f16 || p.k < 8 || (p.k % 8) != 0 || p.n_rows <= 0 || p.stamps == nullptr) return hipErrorInvalidValue;
+    const int blocks = gemv_blocks(p.n_rows);
+    if (n_waves) *n_waves = blocks * kGemvWaves;
+    const size_t lds = (size_t)gemv_iters(p.k, 8) * kWave * 8 * sizeof(float);
+    auto kern = gemv_kernel<half_t, float, kEpiStore, true, kGemvBurst, false, true>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGemvThreads), lds, s, p);
+    return hipGetLastError();
 }
 
 hipError_t launch_gemv(const GemvParams &p, int epilogue, hipStream_t s) {

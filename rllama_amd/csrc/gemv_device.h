@@ -168,8 +168,13 @@ __device__ __forceinline__ void greedy_merge(GreedyBest &g, float ov, int oi, in
 
 // One GEMV over the whole grid: prologue (x staged in LDS), main loop, epilogue.  `smem_raw` is the block's dynamic LDS
 // (gemv_lds_bytes); `red` 16 floats and `rope_f` 64 float2 of static LDS.
-template <typename WT, typename XT, int kEpi, bool kStream, int kPre, int kBurst = kGemvBurst>
+// kEmbed (kEpiRopeKv only): the input row comes from the embedding table (GemvParams::embed_table) instead of p.x.
+// kStamp (measurement builds only): every wavefront records the 100 MHz wall clock at five points into p.stamps.
+constexpr int kGemvStamps = 5; // entry, x staged, first burst consumed, last burst consumed, exit
+template <typename WT, typename XT, int kEpi, bool kStream, int kPre, int kBurst = kGemvBurst, bool kEmbed = false, bool kStamp = false>
 __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw, float *red, float2 *rope_f) {
+    [[maybe_unused]] unsigned long long stamp[kGemvStamps] = {0, 0, 0, 0, 0};
+    if constexpr (kStamp) stamp[0] = wall_clock64();
     using S = GemvShape<WT, kEpi, kBurst>;
     constexpr int kVec = S::kVec, kMats = S::kMats, kRows = S::kRows, kU = S::kU, kPiece = S::kPiece;
     constexpr bool kArgmax = kEpi == kEpiStoreArgmax;
@@ -202,30 +207,38 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     // one table row, widened to f32), named by the token id in the device state: a launch of its own for 16 KB otherwise.
     [[maybe_unused]] const half_t *emb_h = nullptr;
     [[maybe_unused]] const float *emb_f = nullptr;
+    if constexpr (kEmbed) {
+        static_assert(kEpi == kEpiRopeKv, "the embedding row feeds the first product of a token step");
+        const size_t row = (size_t)p.state->token * (size_t)K;
+        if (p.embed_f16) emb_h = reinterpret_cast<const half_t *>(p.embed_table) + row;
+        else emb_f = reinterpret_cast<const float *>(p.embed_table) + row;
+    }
     if constexpr (kEpi == kEpiRopeKv) {
-        if (p.embed_table != nullptr) {
-            const size_t row = (size_t)p.state->token * (size_t)K;
-            if (p.embed_f16) emb_h = reinterpret_cast<const half_t *>(p.embed_table) + row;
-            else emb_f = reinterpret_cast<const float *>(p.embed_table) + row;
-        }
         pos = p.pos1_host > 0 ? p.pos1_host - 1 : p.state->pos;
         const int half_hd = p.head_dim / 2;
         if (tid < half_hd) rope_early = p.freqs[(size_t)pos * half_hd + tid];
     }
-    // four consecutive elements of the input vector
-    auto load_in4 = [&](int i4) -> float4_t {
-        if constexpr (kEpi == kEpiRopeKv) {
+    // one prologue batch of the input vector: kGemvPrologueVecs float4 per thread starting at float4 index `base`; the source is
+    // chosen once, outside the unrolled loads, so that all loads of the batch are issued back to back
+    auto load_batch = [&](int base, int n4, float4_t (&xv)[kGemvPrologueVecs]) {
+        const float4_t *x4 = reinterpret_cast<const float4_t *>(p.x);
+        if constexpr (kEmbed) {
             if (emb_h != nullptr) {
                 typedef __attribute__((ext_vector_type(4))) _Float16 half4_t;
-                const half4_t h = *reinterpret_cast<const half4_t *>(emb_h + (size_t)i4 * 4);
-                return float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+                half4_t hv[kGemvPrologueVecs];
+#pragma unroll
+                for (int j = 0; j < kGemvPrologueVecs; j++) hv[j] = *reinterpret_cast<const half4_t *>(emb_h + (size_t)min(base + tid + j * kGemvThreads, n4 - 1) * 4);
+#pragma unroll
+                for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = float4_t{(float)hv[j][0], (float)hv[j][1], (float)hv[j][2], (float)hv[j][3]};
+                return;
             }
-            if (emb_f != nullptr) return *reinterpret_cast<const float4_t *>(emb_f + (size_t)i4 * 4);
+            if (emb_f != nullptr) x4 = reinterpret_cast<const float4_t *>(emb_f);
         }
-        return reinterpret_cast<const float4_t *>(p.x)[i4];
+#pragma unroll
+        for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = x4[min(base + tid + j * kGemvThreads, n4 - 1)];
     };
     auto load_in1 = [&](int i) -> float {
-        if constexpr (kEpi == kEpiRopeKv) {
+        if constexpr (kEmbed) {
             if (emb_h != nullptr) return (float)emb_h[i];
             if (emb_f != nullptr) return emb_f[i];
         }
@@ -243,8 +256,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
         // RMSNorm::forward (transformer.rs:476-480): (x * rsqrt(mean(x^2) + eps)) * w, x kept in registers
         const float4_t *w4 = reinterpret_cast<const float4_t *>(p.norm_w);
         float4_t xv[kGemvPrologueVecs], av[kGemvPrologueVecs], wv[kGemvPrologueVecs];
-#pragma unroll
-        for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = load_in4(min(tid + j * kGemvThreads, n4 - 1));
+        load_batch(0, n4, xv);
         if (a4 != nullptr) {
 #pragma unroll
             for (int j = 0; j < kGemvPrologueVecs; j++) av[j] = a4[min(tid + j * kGemvThreads, n4 - 1)];
@@ -297,8 +309,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     } else {
         for (int base = 0; base < n4; base += kGemvPrologueVecs * kGemvThreads) {
             float4_t xv[kGemvPrologueVecs], av[kGemvPrologueVecs];
-#pragma unroll
-            for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = load_in4(min(base + tid + j * kGemvThreads, n4 - 1));
+            load_batch(base, n4, xv);
             if (a4 != nullptr) {
 #pragma unroll
                 for (int j = 0; j < kGemvPrologueVecs; j++) av[j] = a4[min(base + tid + j * kGemvThreads, n4 - 1)];
@@ -324,6 +335,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
         if (tid < p.head_dim / 2) rope_f[tid] = rope_early;
     }
     __syncthreads();
+    if constexpr (kStamp) stamp[1] = wall_clock64();
 
     // ---- main loop: row units interleaved over all wavefronts of the grid, so that at any moment the
     //      grid reads one dense window of the matrix ----
@@ -462,8 +474,23 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
                 fetch(unit, c, wv);
             }
             mac(c, wv);
+            if constexpr (kStamp) {
+                // (the products depend on the loaded data, and the clock is read behind them)
+                asm volatile("" : "+v"(acc[0][0]));
+                const unsigned long long now = wall_clock64();
+                if (stamp[2] == 0) stamp[2] = now;
+                stamp[3] = now;
+            }
         }
         finish(unit);
+    }
+    if constexpr (kStamp) {
+        stamp[4] = wall_clock64();
+        if ((threadIdx.x & (kWave - 1)) == 0 && p.stamps != nullptr) {
+            unsigned long long *dst = p.stamps + ((size_t)blockIdx.x * kGemvWaves + threadIdx.x / kWave) * kGemvStamps;
+#pragma unroll
+            for (int i = 0; i < kGemvStamps; i++) dst[i] = stamp[i];
+        }
     }
 
     if constexpr (kArgmax) {

@@ -55,6 +55,7 @@ struct GemvParams {
     int dim;
     int head_dim;
     int max_seq_len;
+    unsigned long long *stamps; // measurement launches only (launch_gemv_stamped): kGemvStamps wall-clock readings per wavefront
     // kEpiStoreArgmax only
     float *amax_ws;           // one 16-byte record per workgroup of the launch (gemv_argmax_ws_bytes)
     unsigned *amax_ticket;    // arrival counter, zero before the launch; the kernel leaves it zero
@@ -68,6 +69,10 @@ hipError_t launch_gemv(const GemvParams &p, int epilogue, hipStream_t s);
 size_t gemv_lds_bytes(int k, int w_is_f16, int x_f16);
 // bytes of GemvParams::amax_ws that any launch can need
 size_t gemv_argmax_ws_bytes();
+// The plain product (kEpiStore, f16 weights, fp32 x) with every wavefront recording the 100 MHz wall clock at kernel entry,
+// when x is staged, behind its first and its last burst, and at exit, into p.stamps [wavefronts of the grid][5]
+// (*n_waves receives their number): where the fixed cost of a launch is spent.
+hipError_t launch_gemv_stamped(const GemvParams &p, hipStream_t s, int *n_waves);
 
 struct AttnDecodeParams {
     const float *q;           // [n_heads x head_dim] f32 (after RoPE)

@@ -136,6 +136,7 @@ extern "C" {
     pub fn rlh_argmax_greedy(logits: *const rlh_tensor, temperature: c_float, token: *mut i32) -> c_int;
     pub fn rlh_model_time_kernel(model: *mut rlh_model, caches: *mut rlh_caches, which: c_int, T: c_int, iters: c_int, us_per_launch: *mut c_float, bytes_per_launch: *mut u64) -> c_int;
     pub fn rlh_time_gemv(ctx: *mut rlh_ctx, rows: c_int, k: c_int, w_dtype: c_int, round_x: c_int, round_y: c_int, n_buffers: c_int, iters: c_int, us_per_launch: *mut c_float) -> c_int;
+    pub fn rlh_probe_gemv_phases(ctx: *mut rlh_ctx, rows: c_int, k: c_int, n_buffers: c_int, launches: c_int, out_us: *mut c_float) -> c_int;
     pub fn rlh_synth_normal_f16(seed: u64, kind: c_int, layer: c_int, first_index: u64, count: u64, std: c_double, out: *mut u16);
     pub fn rlh_synth_tokens(seed: u64, first_index: u64, count: u64, lo: i32, hi: i32, out: *mut i32);
     pub fn rlh_abi_version() -> c_int;
