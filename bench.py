@@ -195,6 +195,86 @@ def other_config_block(ra, ctx, name, warmup=8, kernel_iters=160):
     }
 
 
+def vendor_calibration(ra, ctx) -> int:
+    """Same-box calibration against the vendor library (torch.mm / torch.mv -> hipBLASLt / rocBLAS, f16 in, f16 out): the
+    prompt-path products of the 7B shape at 1024 rows and of the 13B shape at 2048 rows, and the single-row products of the
+    7B shape.  Both sides cycle through enough distinct weight matrices that nothing stays in the 256 MB memory-side cache.
+    torch is used for the vendor side only; nothing of the library depends on it."""
+    import torch
+    rng = np.random.default_rng(0)
+    dev = torch.device("cuda:0")
+
+    def n_copies(n, k):
+        return max(2, int(6e8 // (n * k * 2)) + 1)
+
+    def gemm_pair(m, n, k, iters=24):
+        nb = n_copies(n, k)
+        a = (torch.randn(m, k, device=dev) * 0.1).half()
+        bs = [(torch.randn(n, k, device=dev) * 0.02).half() for _ in range(nb)]
+        for i in range(3 * iters):        # the clocks of an idle part take a few milliseconds of load to come up
+            c = a @ bs[i % nb].t()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(iters):
+            c = a @ bs[i % nb].t()
+        e1.record()
+        torch.cuda.synchronize()
+        vendor = e0.elapsed_time(e1) / iters * 1e3
+        del bs, c
+        A = ra.Tensor.from_numpy(ctx, (rng.standard_normal((m, k)) * 0.1).astype(np.float16))
+        Bs = [ra.Tensor.from_numpy(ctx, ra.synth_normal_f16(7, 5, i, n * k, std=0.02).reshape(n, k)) for i in range(nb)]
+        out = ra.Tensor.zeros(ctx, m, n, ra.TensorDType.Float16)
+        for i in range(3 * iters):
+            ra.check(ctx._lib.rlh_matrix_mul_inplace_transposed(out._h, A._h, Bs[i % nb]._h))
+        ctx.sync()
+        e0 = ctx.event()
+        for i in range(iters):
+            ra.check(ctx._lib.rlh_matrix_mul_inplace_transposed(out._h, A._h, Bs[i % nb]._h))
+        e1 = ctx.event()
+        here = e0.elapsed_ms(e1) / iters * 1e3
+        res = {"vendor_us": round(vendor, 1), "here_us": round(here, 1), "distinct_weight_matrices": nb}
+        if nb >= 2 and n % 8 == 0 and m > 1:
+            for i in range(iters):
+                ra.check(ctx._lib.rlh_ffn_gate(out._h, A._h, Bs[i % nb]._h, Bs[(i + 1) % nb]._h))
+            ctx.sync()
+            e0 = ctx.event()
+            for i in range(iters):
+                ra.check(ctx._lib.rlh_ffn_gate(out._h, A._h, Bs[i % nb]._h, Bs[(i + 1) % nb]._h))
+            e1 = ctx.event()
+            res["two_products_in_one_pass_us"] = round(e0.elapsed_ms(e1) / iters * 1e3, 1)
+        for t in [A, out] + Bs:
+            t.free()
+        return res
+
+    def gemv_pair(n, k, iters=120):
+        nb = n_copies(n, k)
+        ws = [(torch.randn(n, k, device=dev) * 0.02).half() for _ in range(nb)]
+        x = torch.randn(k, device=dev).half()
+        for i in range(2 * iters):
+            y = torch.mv(ws[i % nb], x)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(iters):
+            y = torch.mv(ws[i % nb], x)
+        e1.record()
+        torch.cuda.synchronize()
+        vendor = e0.elapsed_time(e1) / iters * 1e3
+        del ws, y
+        here = ctx.time_gemv(n, k, ra.TensorDType.Float16, False, False, n_buffers=nb, iters=iters)
+        return {"vendor_us": round(vendor, 2), "here_us": round(here, 2), "distinct_weight_matrices": nb}
+
+    out = {"calibration": "vendor library (torch 2.x -> hipBLASLt / rocBLAS) against this library, same box, f16", "gemm": {}, "gemv": {}}
+    for label, (m, d, F) in (("7B shape, 1024 rows", (1024, 4096, 11008)), ("13B shape, 2048 rows", (2048, 5120, 13824))):
+        out["gemm"][label] = {"wq|wk|wv (plain product, no RoPE epilogue)": gemm_pair(m, 3 * d, d), "wo": gemm_pair(m, d, d),
+                              "w1 (one of the pair)": gemm_pair(m, F, d), "w2": gemm_pair(m, d, F)}
+    for n, k in ((4096, 4096), (12288, 4096), (11008, 4096), (22016, 4096), (4096, 11008), (32000, 4096)):
+        out["gemv"][f"{n}x{k}"] = gemv_pair(n, k)
+    print(json.dumps(out))
+    return 0
+
+
 def bench_layer_split(args, ra, ctx, info) -> int:
     """The device's share of a model split by percentage_to_gpu: one prompt call, then K single-token calls of
     rlh_forward_layers, each taking the stream from host memory and returning it there (the hand-off the reference makes at
@@ -263,6 +343,10 @@ def main() -> int:
     ap.add_argument("--percentage-to-gpu", type=float, default=1.0,
                     help="below 1: time the device's share of a layer-split model (rlh_forward_layers over layers "
                          "0..=round(p * (n_layers - 1)), stream handed over from and to host memory on every call)")
+    ap.add_argument("--probe-gemv-phases", action="store_true",
+                    help="run only the wall-clock decomposition of the isolated GEMV launch (rlh_probe_gemv_phases) on the shapes of the 7B model")
+    ap.add_argument("--vendor-calibration", action="store_true",
+                    help="run only the same-box comparison with the vendor library's GEMM / GEMV (needs torch; for profiles/prefill_vendor_calibration.md)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain copy kernel over 1 GiB of f32 (reads 1 GiB, writes 1 GiB per launch): "
                          "the known-size reference for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -274,6 +358,26 @@ def main() -> int:
 
     import rllama_amd as ra
 
+    if args.probe_gemv_phases:
+        ctx = ra.Context(0)
+        out = {"probe": "100 MHz wall clock read by every wavefront at entry, x staged, first burst consumed, last burst consumed, exit; "
+                        "means over 63 back-to-back launches on distinct weight matrices, microseconds", "shapes": {}}
+        for rows, k in ((8, 4096), (2048, 4096), (4096, 4096), (12288, 4096), (11008, 4096), (4096, 11008), (32000, 4096)):
+            nb = min(24, max(2, int(1.2e9 // (rows * k * 2)) + 1))
+            r = ctx.probe_gemv_phases(rows, k, n_buffers=nb, launches=64)
+            r["hip_event_us_per_launch"] = round(ctx.time_gemv(rows, k, ra.TensorDType.Float16, False, False, n_buffers=nb, iters=200), 2)
+            r["weight_bytes"] = rows * k * 2
+            out["shapes"][f"{rows}x{k}"] = r
+        ctx.close()
+        print(json.dumps(out))
+        return 0
+    if args.vendor_calibration:
+        import torch  # before the library's own context: torch brings its own copy of the HIP runtime and wants to be first
+        torch.zeros(1, device="cuda:0")
+        ctx = ra.Context(0)
+        rc = vendor_calibration(ra, ctx)
+        ctx.close()
+        return rc
     if args.calibrate_copy:
         ctx = ra.Context(0)
         rows, cols = 16384, 16384  # 2^28 f32 = 1 GiB

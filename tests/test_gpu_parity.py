@@ -539,6 +539,34 @@ def test_config0_f32_mode_end_to_end(ctx):
     gm.free()
 
 
+def test_set_option_names_and_values(ctx):
+    """rlh_set_option: the switches rlh_init reads from RLLAMA_HIP_<NAME> once, changed per context afterwards; unknown names
+    and unusable values are refused and leave the switch as it was."""
+    for name, good, bad in (("GEMM_DUAL", "3", "9"), ("ATTN_MERGE", "0", "1"), ("ATTN_CHUNK", "64", "5"), ("GEMM_TILE", "2", "7"),
+                            ("PREFILL_ATTN", "gemm", "whatever"), ("PREFILL_ATTN_ORDER", "1", "3")):
+        ctx.set_option(name, good)
+        with pytest.raises(rllama_amd.RllamaHipError) as ei:
+            ctx.set_option(name, bad)
+        assert ei.value.code == 1 and name in str(ei.value)
+        ctx.set_option(name, None)
+    for name in ("NO_SUCH_SWITCH", "FUSED", "GEMM_SIMPLE", ""):
+        with pytest.raises(rllama_amd.RllamaHipError):
+            ctx.set_option(name, "1")
+    # a switch takes effect on the next call of an existing model and goes back with None: the split attention merged by a
+    # second launch and inside the kernel give the same bits (the same partial results, added in the same order)
+    shape = Shape(dim=128, n_layers=1, n_heads=2, ffn_hidden=256, vocab_size=64, max_seq_len=600)
+    gm = make_gpu(ctx, shape, synth_weights(shape, seed=9, std=0.08), True)
+    toks = np.random.default_rng(10).integers(0, 64, 500)
+    c = gm.make_caches()
+    gm.forward(toks, 0, c)
+    c2 = c.true_clone()
+    a = gm.forward([5], 500, c)
+    with options(ctx, ATTN_MERGE="0", ATTN_CHUNK="64"):
+        b = gm.forward([5], 500, c2)
+    assert np.array_equal(gm.forward([7], 501, c), gm.forward([7], 501, c2)) and max_rel_err(a, b) < 1e-3
+    gm.free()
+
+
 def test_cache_services_and_errors(ctx):
     shape = TINY
     W = synth_weights(shape, seed=31, std=0.1)
