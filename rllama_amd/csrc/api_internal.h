@@ -42,7 +42,7 @@ constexpr int kOpMaxHeads = 1024;
 struct Tunables {
     rlh::GemmTune gemm{};
     int gemv_burst_fixed = 0;      // GEMV_BURST=0: single-row products always issue bursts of 8 loads per lane
-    int attn_chunk = 0;            // ATTN_CHUNK=N (>= 16): positions per workgroup of a split sequence; 0 = one workgroup per compute unit
+    int attn_chunk = -1;           // ATTN_CHUNK: positions per workgroup of a split sequence: N >= 16, 0 = 128, -1 = about one workgroup per compute unit
     int attn_single_max = 384;     // ATTN_SINGLE_MAX=N: longest sequence one workgroup per head handles alone
     int attn_merge_mode = 2;       // ATTN_MERGE=0: the pieces of a split sequence are combined by a second launch; 2: inside the kernel
     int attn_lds = 0;              // ATTN_LDS=1: cache rows staged through LDS (comparison form)

@@ -366,9 +366,12 @@ extern "C" int rlh_rope_kvwrite(rlh_tensor *q, const rlh_tensor *k, const rlh_te
 
 namespace rlh {
 int attn_splits_rule(int T, int n_heads, int compute_units, int single_max, int chunk, int max_splits) {
-    // One workgroup per (head, split).  Short sequences stay in one workgroup per head; longer ones are cut into pieces of
-    // about `chunk` positions (chunk > 0), or of kAutoChunk positions (chunk == 0, the default), or so that the part holds
-    // about one workgroup per compute unit, in pieces of at least 128 positions (chunk == -1).
+    // One workgroup per (head, split).  Short sequences stay in one workgroup per head; longer ones are cut so that the part
+    // holds about one workgroup per compute unit, in pieces of at least 128 positions (chunk == -1, the default), or into
+    // pieces of about `chunk` positions (chunk > 0; chunk == 0: 128).  Measured at 2112 positions of the 13B shape (40 heads):
+    // 6 pieces of 352 positions 13.0 - 14.0 us, 17 of 128 14.1 - 14.5 us -- every piece ends at about the same time, and the
+    // workgroup that merges loads 6 partial results instead of 17; the 7B shape (32 heads) gets the same pieces up to 1024
+    // positions and 8 of 256 instead of 16 of 128 at 2048 (12.25 against 12.35 us).
     constexpr int kAutoChunk = 128;
     if (T <= single_max) return 1;
     int S;
