@@ -103,9 +103,10 @@ static hipError_t launch_gemv_e(const GemvParams &p, hipStream_t s) {
     return p.x_f16 ? launch_gemv_t<float, half_t, kEpi>(p, s) : launch_gemv_t<float, float, kEpi>(p, s);
 }
 
-hipError_t launch_gemv_stamped(const GemvParams &p, hipStream_t s, int *n_waves) {
+hipError_t launch_gemv_stamped(const GemvParams &p, hipStream_t s, int stamps_capacity_waves, int *n_waves) {
     if (!p.w_is_f16 || p.x_f16 || p.k < 8 || (p.k % 8) != 0 || p.n_rows <= 0 || p.stamps == nullptr) return hipErrorInvalidValue;
     const int blocks = gemv_blocks(p.n_rows);
+    if (blocks * kGemvWaves > stamps_capacity_waves) return hipErrorInvalidValue; // every wavefront writes its stamps: checked before the launch
     if (n_waves) *n_waves = blocks * kGemvWaves;
     const size_t lds = (size_t)gemv_iters(p.k, 8) * kWave * 8 * sizeof(float);
     auto kern = gemv_kernel<half_t, float, kEpiStore, true, kGemvBurst, false, true>;

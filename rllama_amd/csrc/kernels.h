@@ -72,7 +72,7 @@ size_t gemv_argmax_ws_bytes();
 // The plain product (kEpiStore, f16 weights, fp32 x) with every wavefront recording the 100 MHz wall clock at kernel entry,
 // when x is staged, behind its first and its last burst, and at exit, into p.stamps [wavefronts of the grid][5]
 // (*n_waves receives their number): where the fixed cost of a launch is spent.
-hipError_t launch_gemv_stamped(const GemvParams &p, hipStream_t s, int *n_waves);
+hipError_t launch_gemv_stamped(const GemvParams &p, hipStream_t s, int stamps_capacity_waves, int *n_waves);
 
 struct AttnDecodeParams {
     const float *q;           // [n_heads x head_dim] f32 (after RoPE)

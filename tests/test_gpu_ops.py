@@ -357,3 +357,21 @@ def test_device_greedy_pick_full_vocab_and_odd_sizes(ctx):
             logits = (rng.standard_normal(V) * 4.0).astype(f32)
             want, _, _ = oracle.sample_greedy(logits, 1.0)
             assert Tensor.from_numpy(ctx, logits.reshape(-1, 1)).argmax_greedy() == want
+
+
+def test_gemv_phase_probe_reads_a_consistent_clock(ctx):
+    """rlh_probe_gemv_phases (measurement only): the wall-clock readings inside the kernel are ordered as the kernel runs --
+    every phase non-negative and shorter than the launch it belongs to, the launch as the device sees it no longer than what
+    HIP events measure around it plus the gap in front -- and bad arguments are refused."""
+    rows, k = 2048, 4096
+    r = ctx.probe_gemv_phases(rows, k, n_buffers=4, launches=16)
+    assert set(r) == set(rllama_amd.Context.GEMV_PHASES) and all(np.isfinite(v) and v >= 0.0 for v in r.values()), r
+    whole = r["first_entry_to_last_exit"]
+    assert 1.0 < whole < 200.0, r
+    for name in ("dispatch_ramp", "prologue", "first_byte_latency", "streaming", "epilogue", "tail_skew"):
+        assert r[name] <= whole, (name, r)
+    events = ctx.time_gemv(rows, k, TensorDType.Float16, False, False, n_buffers=4, iters=50)
+    assert whole + r["gap_after_previous_launch"] < 3.0 * events + 5.0, (r, events)     # stamps cost a little; same order of magnitude
+    for bad in ((0, k, 4, 16), (rows, 12, 4, 16), (rows, k, 0, 16), (rows, k, 4, 1)):
+        with pytest.raises(rllama_amd.RllamaHipError):
+            ctx.probe_gemv_phases(bad[0], bad[1], n_buffers=bad[2], launches=bad[3])
