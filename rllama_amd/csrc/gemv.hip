@@ -36,9 +36,15 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     extern __shared__ uint4_t smem_raw[];
     __shared__ float red[16];
     __shared__ float2 rope_f[64]; // (cos, sin) of this position, head_dim / 2 <= 64 entries
-    // (measured: issuing the first burst behind the prologue's loads is worth 1 % on the w1|w3 product, nothing or a loss on
-    // the others, so only that instantiation does it)
-    constexpr int kPre = (RLH_GEMV_PRELOAD && kEpi == kEpiSilu) ? kPreSelf : kPreNone;
+    // The first burst of weights is issued right behind the prologue's own loads (behind those of its last batch where x takes
+    // more than one), so that its memory latency runs under the norm / staging work while x stays ahead of it in the in-order
+    // return queue, and is consumed in front of the main loop.  Measured per launch against the same kernel without it --
+    // 7B shape: wq|wk|wv 19.3 -> 18.9 us, wo 8.05 -> 8.0, w2 17.1 -> 16.4, the isolated 11008 x 4096 product 16.3 -> 15.9,
+    // 4096 x 11008 17.6 -> 16.9; 13B shape: wq|wk|wv 27.3 -> 27.05, wo 10.8 -> 10.6, w2 24.3 -> 24.15; w1|w3 has done it since
+    // it was worth 1.6 % there.  (Issued behind the first of w2's two batches of x it cost 0.4 us instead: the second batch
+    // waits behind the burst.  With a test for it inside the main loop the 13B wq|wk|wv lost 0.6 us.)  The output head with the
+    // greedy pick gains nothing from it and does not do it.
+    constexpr int kPre = ((RLH_GEMV_PRELOAD_EPIS >> kEpi) & 1) ? kPreSelf : kPreNone;
     gemv_body<WT, XT, kEpi, kStream, kPre, kBurst, kEmbed, kStamp>(p, smem_raw, red, rope_f);
 }
 

@@ -34,8 +34,8 @@ constexpr int kGemvWaves = RLH_GEMV_WAVES;
 constexpr int kGemvThreads = kGemvWaves * kWave;
 constexpr int kGemvTargetWaves = RLH_GEMV_TARGET_WAVES;
 constexpr int kGemvBurst = RLH_GEMV_BURST; // 16-byte loads per lane issued back to back before they are consumed
-#ifndef RLH_GEMV_PRELOAD
-#define RLH_GEMV_PRELOAD 1
+#ifndef RLH_GEMV_PRELOAD_EPIS
+#define RLH_GEMV_PRELOAD_EPIS 0x0d // bit per epilogue (kEpiStore, kEpiRopeKv, kEpiSilu): its first burst is issued by the prologue
 #endif
 #ifndef RLH_GEMV_PROLOGUE_VECS
 #define RLH_GEMV_PROLOGUE_VECS 8
@@ -316,7 +316,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
 #pragma unroll
                 for (int j = 0; j < kGemvPrologueVecs; j++) xv[j] = xv[j] + av[j];
             }
-            if (base == 0) {
+            if (base + kGemvPrologueVecs * kGemvThreads >= n4) { // behind the loads of the last batch: x stays ahead of it in the return queue
                 __builtin_amdgcn_sched_barrier(0);
                 preload();
             }
@@ -460,23 +460,34 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     // unit before, so that the partial last round of units -- 768 of 2048 wavefronts on the 7B shape's 11008 rows -- costs no
     // memory latency of its own: the isolated 11008 x 4096 product 16.45 -> 17.25 us, w1|w3 30.1 -> 30.6 us, and with the code
     // in place but switched off w2 17.1 -> 17.7 us.)
-    for (int unit = unit_first; unit < n_units; unit += W) {
+    // The burst the prologue requested (pieces 0 .. kU - 1 of the first row unit) is consumed in front of the loop, so that
+    // the loop itself carries no test for it.
 #pragma unroll
-        for (int m = 0; m < kMats; m++)
+    for (int m = 0; m < kMats; m++)
 #pragma unroll
-            for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
-        for (int c = 0; c < pieces; c += kU) {
+        for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
+    int c_first = 0;
+    if constexpr (kPre != kPreNone) {
+        if (have_pre) {
             uint4_t wv[kU][kMats][kRows];
-            if (kPre != kPreNone && have_pre && c == 0 && unit == unit_first) {
 #pragma unroll
-                for (int u = 0; u < kU; u++)
+            for (int u = 0; u < kU; u++)
 #pragma unroll
-                    for (int m = 0; m < kMats; m++)
+                for (int m = 0; m < kMats; m++)
 #pragma unroll
-                        for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[(u * kMats + m) * kRows + r];
-            } else {
-                fetch(unit, c, wv);
+                    for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[(u * kMats + m) * kRows + r];
+            mac(0, wv);
+            c_first = kU;
+            if constexpr (kStamp) {
+                asm volatile("" : "+v"(acc[0][0]));
+                stamp[2] = stamp[3] = wall_clock64();
             }
+        }
+    }
+    for (int unit = unit_first; unit < n_units; unit += W) {
+        for (int c = c_first; c < pieces; c += kU) {
+            uint4_t wv[kU][kMats][kRows];
+            fetch(unit, c, wv);
             mac(c, wv);
             if constexpr (kStamp) {
                 // (the products depend on the loaded data, and the clock is read behind them)
@@ -487,6 +498,11 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
             }
         }
         finish(unit);
+        c_first = 0;
+#pragma unroll
+        for (int m = 0; m < kMats; m++)
+#pragma unroll
+            for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
     }
     if constexpr (kStamp) {
         stamp[4] = wall_clock64();
