@@ -44,7 +44,8 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(GemvParams p) {
     // it was worth 1.6 % there.  (Issued behind the first of w2's two batches of x it cost 0.4 us instead: the second batch
     // waits behind the burst.  With a test for it inside the main loop the 13B wq|wk|wv lost 0.6 us.)  The output head with the
     // greedy pick gains nothing from it and does not do it.
-    constexpr int kPre = ((RLH_GEMV_PRELOAD_EPIS >> kEpi) & 1) ? kPreSelf : kPreNone;
+    // (The stamped measurement build keeps the burst behind the prologue, so that "x staged" and "first burst" stay two phases.)
+    constexpr int kPre = (!kStamp && ((RLH_GEMV_PRELOAD_EPIS >> kEpi) & 1)) ? kPreSelf : kPreNone;
     gemv_body<WT, XT, kEpi, kStream, kPre, kBurst, kEmbed, kStamp>(p, smem_raw, red, rope_f);
 }
 
