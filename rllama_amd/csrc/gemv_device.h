@@ -37,6 +37,13 @@ constexpr int kGemvBurst = RLH_GEMV_BURST; // 16-byte loads per lane issued back
 #ifndef RLH_GEMV_PRELOAD_EPIS
 #define RLH_GEMV_PRELOAD_EPIS 0x0d // bit per epilogue (kEpiStore, kEpiRopeKv, kEpiSilu): its first burst is issued by the prologue
 #endif
+#ifndef RLH_GEMV_AHEAD_EPIS
+#define RLH_GEMV_AHEAD_EPIS 0x11 // bit per epilogue (kEpiStore, kEpiStoreArgmax): the next row unit's first burst is requested in
+                                 // front of the current unit's reduction and epilogue.  Measured per launch: wo of the 7B shape
+                                 // 8.0 -> 7.55 us, of the 13B shape 10.7 -> 10.2, the isolated 11008 x 4096 product 16.0 -> 15.6,
+                                 // the head 41.3 -> 40.8; w2 unchanged; wq|wk|wv and w1|w3 unchanged at the 7B shape and 0.4 us
+                                 // slower at the 13B shape, so they do not do it.
+#endif
 #ifndef RLH_GEMV_PROLOGUE_VECS
 #define RLH_GEMV_PROLOGUE_VECS 8
 #endif
@@ -460,31 +467,33 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
     // unit before, so that the partial last round of units -- 768 of 2048 wavefronts on the 7B shape's 11008 rows -- costs no
     // memory latency of its own: the isolated 11008 x 4096 product 16.45 -> 17.25 us, w1|w3 30.1 -> 30.6 us, and with the code
     // in place but switched off w2 17.1 -> 17.7 us.)
-    // The burst the prologue requested (pieces 0 .. kU - 1 of the first row unit) is consumed in front of the loop, so that
-    // the loop itself carries no test for it.
+    // The burst the prologue requested (pieces 0 .. kU - 1 of the first row unit) is consumed at the head of that unit.  With
+    // kAhead the first burst of the *next* unit is requested before the reduction and epilogue of the current one run, so
+    // that those run under its memory latency.
+    constexpr bool kAhead = !kStamp && ((RLH_GEMV_AHEAD_EPIS >> kEpi) & 1);
+    const bool burst0_full = kU <= pieces_full;
+    bool have = false;
+    if constexpr (kPre != kPreNone) have = have_pre;
+    for (int unit = unit_first; unit < n_units; unit += W) {
 #pragma unroll
-    for (int m = 0; m < kMats; m++)
+        for (int m = 0; m < kMats; m++)
 #pragma unroll
-        for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
-    int c_first = 0;
-    if constexpr (kPre != kPreNone) {
-        if (have_pre) {
-            uint4_t wv[kU][kMats][kRows];
+            for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
+        int c_first = 0;
+        if constexpr (kPre != kPreNone || kAhead) {
+            if (have) {
+                uint4_t wv[kU][kMats][kRows];
 #pragma unroll
-            for (int u = 0; u < kU; u++)
+                for (int u = 0; u < kU; u++)
 #pragma unroll
-                for (int m = 0; m < kMats; m++)
+                    for (int m = 0; m < kMats; m++)
 #pragma unroll
-                    for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[(u * kMats + m) * kRows + r];
-            mac(0, wv);
-            c_first = kU;
-            if constexpr (kStamp) {
-                asm volatile("" : "+v"(acc[0][0]));
-                stamp[2] = stamp[3] = wall_clock64();
+                        for (int r = 0; r < kRows; r++) wv[u][m][r] = wpre[(u * kMats + m) * kRows + r];
+                mac(0, wv);
+                c_first = kU;
+                have = false;
             }
         }
-    }
-    for (int unit = unit_first; unit < n_units; unit += W) {
         for (int c = c_first; c < pieces; c += kU) {
             uint4_t wv[kU][kMats][kRows];
             fetch(unit, c, wv);
@@ -497,12 +506,22 @@ __device__ __forceinline__ void gemv_body(const GemvParams &p, uint4_t *smem_raw
                 stamp[3] = now;
             }
         }
+        if constexpr (kAhead) {
+            const int next = unit + W;
+            if (next < n_units && burst0_full) {
+#pragma unroll
+                for (int u = 0; u < kU; u++)
+#pragma unroll
+                    for (int m = 0; m < kMats; m++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++)
+                            wpre[(u * kMats + m) * kRows + r] =
+                                load16<kStream>(wmat[m] + (size_t)(next * kRows + r) * K + (size_t)u * kPiece + lane * kVec);
+                have = true;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
         finish(unit);
-        c_first = 0;
-#pragma unroll
-        for (int m = 0; m < kMats; m++)
-#pragma unroll
-            for (int r = 0; r < kRows; r++) acc[m][r] = 0.0f;
     }
     if constexpr (kStamp) {
         stamp[4] = wall_clock64();
