@@ -160,6 +160,13 @@ __global__ __launch_bounds__(kThreads) void attn_decode_kernel(AttnDecodeParams 
                     const int r = min(t + u * stride, t_safe) - t0;
                     kraw[u][w] = lds_k[r * kLanesPerPos + dl];
                     vraw[u][w] = lds_v[r * kLanesPerPos + dl];
+                } else if (kAttnBatch == 8 && !(t + u * stride < t1)) {
+                    // The single batch of 8 steps (129 .. 256 positions per block): positions past the end request nothing.
+                    // One workgroup per head is bound by what its compute unit can take in, and a clamped load costs as
+                    // much of that as a real one: 4.77 -> 4.41 us at 136 positions of the 7B shape, 4.85 -> 4.55 at 160.
+                    // (In the looping forms the same test cost 0.1 - 0.3 us per launch, so they keep the clamped loads.)
+                    kraw[u][w] = uint4_t{0u, 0u, 0u, 0u};
+                    vraw[u][w] = uint4_t{0u, 0u, 0u, 0u};
                 } else {
                     kraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(kbase + off) + 16 * w);
                     vraw[u][w] = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(vbase + off) + 16 * w);
