@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the dominant kernel (c1: w13 GEMV; c3: w1-shape GEMM; 7B shapes).  These are RECORDED values, not
 # something a bench run measures: they come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same script, each scaled
 # by the same counter on a 1 GiB copy kernel; the summaries named here hold the commands and the raw counter readings.
-MEASURED_TRAFFIC = {"c1": 180_986_300, "c3": 284_171_967}
+MEASURED_TRAFFIC = {"c1": 180_986_026, "c3": 284_149_621}
 TRAFFIC_SOURCE = {"c1": "profiles/decode_c1_hbm_traffic_pmc.md", "c3": "profiles/prefill_c3_hbm_traffic_pmc.md"}
 
 CONFIGS = {
